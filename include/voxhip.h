@@ -365,10 +365,15 @@ int vox_lm_prefill(vox_lm* m, void* stream, const vox_lm_io* io, const int32_t* 
  * (prompt portions next to single decoded tokens); rows of a request are contiguous and ascending in position.      */
 typedef struct vox_hybrid vox_hybrid;
 enum { VOX_MIXER_HGRN2 = 0, VOX_MIXER_POOLED_WINDOW_ATTN = 1, VOX_MIXER_MLSTM = 2, VOX_MIXER_RGLRU = 3, VOX_MIXER_CAUSAL_ATTN = 4,
-       VOX_MIXER_SHIFT_DECAY = 5 };
+       VOX_MIXER_SHIFT_DECAY = 5, VOX_MIXER_LATENT_ATTN = 6, VOX_MIXER_RETENTION = 7 };
 enum { VOX_HYBRID_BF16 = 0, VOX_HYBRID_F32 = 1 };
 enum { VOX_NORM_LAYER = 0 /* weight-only layer norm */, VOX_NORM_RMS_GROUPS = 1 /* RMS norm over norm_groups equal slices */ };
-enum { VOX_BLOCK_SEQUENTIAL = 0, VOX_BLOCK_PARALLEL = 1 };
+/* sequential: x += mixer(norm1 x); x += ff(norm2 x).  parallel: x += mixer(norm1 x) + ff(norm2 x).  parallel, one norm:
+ * x += mixer(n) + ff(n) with n = norm1 x (norm2 is not used) */
+enum { VOX_BLOCK_SEQUENTIAL = 0, VOX_BLOCK_PARALLEL = 1, VOX_BLOCK_PARALLEL_ONE_NORM = 2 };
+enum { VOX_FF_UP_DOWN = 0 /* down(gelu_erf(up h)) */, VOX_FF_GATED = 1 /* down(act(gate h + b) * (up h + b)) + b */ };
+enum { VOX_ACT_GELU_TANH = 0, VOX_ACT_SWISH = 1 /* g * sigmoid(alpha g) */ };
+enum { VOX_ROUTER_SOFTMAX = 0, VOX_ROUTER_SIGMOID = 1 };
 /* Routed feed-forward.  Router logits z = router . h in fp32; s = softmax(z) over experts + identity outputs; the `top`
  * largest of s + correction are chosen; their weights are s / (sum of the chosen s + 1e-20).  Expert e < experts:
  * g = min(gate_e h, limit), u = clamp(up_e h, -limit, limit), y = g * sigmoid(act_alpha * g) * (u + 1), output down_e y.
@@ -382,6 +387,8 @@ typedef struct {
     const void* w_down;           /* [experts][width][ff] */
     const void* shared_gate_up;   /* [2*shared_ff][width] */
     const void* shared_down;      /* [width][shared_ff] */
+    int32_t score_kind, renorm, scale_input;
+    float up_offset;
 } vox_hybrid_moe;
 typedef struct {
     int32_t kind, heads, kv_heads, dim, vdim;
@@ -427,13 +434,34 @@ typedef struct {
     const void* w_decay2;                 /* [heads*dim, lora] engine dtype */
     const float *decay0, *bonus;          /* [heads*dim] fp32 each */
     const vox_hybrid_moe* moe;            /* routed feed-forward or NULL */
+    /* dense feed-forward form: VOX_FF_GATED keeps gate rows, then up rows in w_up [2*ff, width], biases b_up [2*ff] and b_down [width]
+     * (fp32 or NULL) and the activation ff_act (VOX_ACT_*, swish with slope 1) */
+    int32_t ff_kind, ff_act;
+    const float *b_up, *b_down;
+    /* latent attention (heads of `dim` plain + rot_dim rotated query / key dims, values of vdim): w_in rows = query latent (q_rank) |
+     * key / value latent (kv_rank) | shared rotated key part (rot_dim) | output gate (heads).  Both latents are RMS-normed with a weight
+     * (q_lat_norm, kv_lat_norm).  q = w_uq (normed query latent), per head [dim plain | rot_dim rotated]; per head the plain key is
+     * w_uk (latent) and the value w_uv (latent).  score = (q_plain . k_plain + q_rot . k_rot) * scale over the last `window` tokens
+     * (0: all), softmax, each head's output times sigmoid of its gate.  The cache keeps the normed latent and the rotated key part
+     * only: scores are taken against the latent with w_uk folded into the query (w_ukT), values expanded after the weighted sum.
+     * Rotation of the new kinds: dims i and i + rot_dims/2 of the rotated vector form a pair (angle = position * inv_freq[i]). */
+    int32_t q_rank, kv_rank, rot_dim;
+    const void* w_uq;                     /* [heads*(dim+rot_dim), q_rank] */
+    const void* w_ukT;                    /* [heads][kv_rank][dim]: per head the transpose of its rows of w_uk */
+    const void* w_uv;                     /* [heads*vdim, kv_rank] */
+    const float *q_lat_norm, *kv_lat_norm;
+    /* retention: w_in rows = q (heads*dim) | k (heads*dim) | v (heads*vdim) | gate (heads*vdim); q, k rotated on their first rot_dims
+     * dims, k then times dim^-1/2; S <- decay[h] S + k v^T, o = S^T q; unit RMS per head (weight head_norm [heads*vdim] or none),
+     * times silu(gate) */
+    const float* decay;                   /* [heads] fp32 */
 } vox_hybrid_layer;
 typedef struct {
     int32_t layer;       /* index into layers */
     int32_t loop_in;     /* 1: x <- loop_in [x; x0] before this run */
-    void* cache;         /* attention: K [max_pages*page_size][kv_heads*dim] then V [max_pages*page_size][kv_heads*vdim], engine dtype */
+    void* cache;         /* attention: K [max_pages*page_size][kv_heads*dim] then V [max_pages*page_size][kv_heads*vdim], engine dtype;
+                            latent attention: [max_pages*page_size][kv_rank + rot_dim] */
     float* pool;         /* pooled attention: [max_pages][(page_size-1)/pool+1][kv_heads][dim+vdim] */
-    /* HGRN2: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1]; RGLRU: [slots][conv_taps][C] (S, then the last
+    /* HGRN2, retention: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1]; RGLRU: [slots][conv_taps][C] (S, then the last
      * conv_taps-1 inputs of the convolution, oldest first); shift-decay: [slots][heads*dim*dim + width] (S, then the previous
      * token's normed input) */
     float* state;
@@ -446,12 +474,17 @@ typedef struct {
     float eps;
     int32_t norm_kind, norm_groups;       /* VOX_NORM_*; slices of the grouped RMS norm (>= 1) */
     float embed_scale;                    /* x0 = embedding[id] * embed_scale */
+    float logit_softcap;                  /* > 0: logits <- cap * tanh(logits / cap) */
+    /* bigram_buckets > 0: x0 += bigram[(prev * bigram_mul_prev + id * bigram_mul_cur) mod buckets], row `buckets` for a sequence's first token */
+    int32_t bigram_buckets, bigram_mul_prev, bigram_mul_cur;
 } vox_hybrid_config;
 typedef struct {
     const vox_hybrid_layer* layers;
     const vox_hybrid_run* runs;
     const void *embedding /*[vocab,width]*/, *loop_in /*[width,2*width] or NULL*/, *head /*[vocab,width]*/;
     const float* final_norm;
+    const void* bigram;                   /* [bigram_buckets + 1, width] or NULL */
+    int32_t* prev_token;                  /* state, [slots]: the last token each slot's sequence has seen (bigram embedding) */
 } vox_hybrid_weights;
 typedef struct {
     const int32_t *pos, *row_req, *page, *slot;   /* per row: position, request index in this step, K/V page and slot */

@@ -44,9 +44,10 @@ template <typename T> __device__ __forceinline__ float hb_operand(float v);
 template <> __device__ __forceinline__ float hb_operand<float>(float v) { return v; }
 template <> __device__ __forceinline__ float hb_operand<bf16_t>(float v) { return bfround(v); }
 
-// A lane-chunked dot product in k_hb_gemv's order: chunks of CH at lane*CH + 64*CH*i, then a butterfly.
+// A lane-chunked dot product in k_hb_gemv's order: chunks of CH at lane*CH + 64*CH*i, then a butterfly.  xs multiplies x before it
+// becomes an operand.
 template <typename T>
-__device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, bool vec, int lane) {
+__device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, bool vec, int lane, float xs = 1.0f) {
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     float a = 0.f;
     if (vec) {
@@ -61,18 +62,20 @@ __device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, 
                 wv[0] = u.x; wv[1] = u.y; wv[2] = u.z; wv[3] = u.w;
             }
 #pragma unroll
-            for (int i = 0; i < CH; ++i) a = fmaf(wv[i], hb_operand<T>(x[k + i]), a);
+            for (int i = 0; i < CH; ++i) a = fmaf(wv[i], hb_operand<T>(x[k + i] * xs), a);
         }
     } else {
-        for (int k = lane; k < K; k += 64) a = fmaf(hb_ld(w + k), hb_operand<T>(x[k]), a);
+        for (int k = lane; k < K; k += 64) a = fmaf(hb_ld(w + k), hb_operand<T>(x[k] * xs), a);
     }
     return hb_wave_sum(a);
 }
-enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3 };
-template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias) {
+// HB_EPI_SOFTCAP: v <- arg * tanh(v / arg) (arg = the product's hb_rowmap::epi_arg)
+enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3, HB_EPI_SOFTCAP = 4 };
+template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias, float arg = 0.f) {
     float v = acc + bias;
     if (EPI == HB_EPI_GELU) v = 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
     if (EPI == HB_EPI_TANH) v = tanhf(v);
+    if (EPI == HB_EPI_SOFTCAP) v = arg * tanhf(v / arg);
     if (EPI == HB_EPI_RESID) v = *c + v;
     *c = v;
 }
@@ -82,28 +85,57 @@ __device__ __forceinline__ float hb_gelu_tanh(float z) {
 // Several products in one launch: product z uses the matrix Wt + z*w_stride, the activations A + z*a_stride, the outputs
 // C + z*c_stride and the bias + z*b_stride (a strided batch: block-diagonal matrices, projections that each read their own input).
 // count != NULL (routed experts): product z takes the gathered rows list[z*cap + 0 .. count[z]); the A row of list entry v is
-// v / a_div, its C row is v.
+// v / a_div, its C row is v; a_scale != NULL: the A row of entry v is multiplied by a_scale[v] before it becomes an operand.
 struct hb_rowmap {
     const int* count;
     const int* list;
     int cap, a_div;
     long w_stride, a_stride, c_stride, b_stride;
+    const float* a_scale;
+    float epi_arg;
 };
-static inline hb_rowmap hb_plain() { return hb_rowmap{nullptr, nullptr, 0, 1, 0, 0, 0, 0}; }
+static inline hb_rowmap hb_plain() { return hb_rowmap{nullptr, nullptr, 0, 1, 0, 0, 0, 0, nullptr, 0.f}; }
 
 // ---- embedding gather: x[row] = table[id]; the second half of both residual buffers keeps the embedding output ----------
+// A bigram table (bg.table != NULL) adds row (prev * mul_prev + id * mul_cur) mod buckets, prev being the token before this one in its
+// sequence: the previous row of the request, or what the request's state slot remembers, or nothing at position 0 (row `buckets`).
+// Steps with one row per request (bg.store) also leave the row's id in the slot; other steps do that in k_hb_store_prev, after every
+// block of this launch has read its predecessor.
+struct hb_bigram {
+    const void* table;
+    int* prev;              // [slots]
+    int buckets, mul_prev, mul_cur, store;
+};
+__device__ __forceinline__ int hb_clamp_id(int id, int vocab) { return id < 0 ? 0 : (id >= vocab ? vocab - 1 : id); }
 template <typename T>
 __global__ __launch_bounds__(256) void k_hb_embed(const T* table, const int* ids, int id_stride, float* xa, float* xb, int W, int vocab,
-                                                  float scale) {
+                                                  float scale, hb_bigram bg, const int* pos, const int* row_req, const int* req_rows,
+                                                  const int* req_state) {
     const int row = blockIdx.x;
-    int id = ids[(size_t)row * id_stride];
-    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const int id = hb_clamp_id(ids[(size_t)row * id_stride], vocab);
+    const T* extra = nullptr;
+    if (bg.table) {
+        const int r = row_req[row];
+        long b = bg.buckets;
+        if (pos[row] > 0) {
+            const int before = row > req_rows[r] ? hb_clamp_id(ids[(size_t)(row - 1) * id_stride], vocab) : bg.prev[req_state[r]];
+            b = ((long)before * bg.mul_prev + (long)id * bg.mul_cur) % bg.buckets;
+        }
+        extra = (const T*)bg.table + (size_t)b * W;
+        __syncthreads();        // (one row per request: the slot is read above by every thread before thread 0 replaces it)
+        if (bg.store && threadIdx.x == 0) bg.prev[req_state[r]] = id;
+    }
     for (int i = threadIdx.x; i < W; i += 256) {
-        const float v = hb_ld(table + (size_t)id * W + i) * scale;
+        float v = hb_ld(table + (size_t)id * W + i) * scale;
+        if (extra) v += hb_ld(extra + i);
         xa[(size_t)row * 2 * W + i] = v;
         xa[(size_t)row * 2 * W + W + i] = v;
         xb[(size_t)row * 2 * W + W + i] = v;
     }
+}
+__global__ void k_hb_store_prev(const int* ids, int id_stride, int vocab, const int* req_rows, const int* req_state, int* prev, int n_req) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < n_req && req_rows[r + 1] > req_rows[r]) prev[req_state[r]] = hb_clamp_id(ids[(size_t)(req_rows[r + 1] - 1) * id_stride], vocab);
 }
 
 // ---- layer norm with a weight and no bias, fp32; optional row gather ----------------------------------------------------
@@ -245,10 +277,12 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
     float4 ra[NA];
     uint4 rw[2];
     const float* arow[NA];
+    float asc[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
         const int gm = m0 + ((tid + i * 256) >> 4);
         arow[i] = gm < M ? A + (size_t)(lst ? lst[gm] / rm.a_div : gm) * lda : nullptr;
+        asc[i] = gm < M && lst && rm.a_scale ? rm.a_scale[lst[gm]] : 1.0f;
     }
     auto fetch = [&](int k0) {
         // A tile: BM x 64 fp32
@@ -294,8 +328,8 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
         for (int i = 0; i < NA; ++i) {
             const int idx = tid + i * 256;
             uint2 o;
-            o.x = pack_bf2(ra[i].x, ra[i].y);
-            o.y = pack_bf2(ra[i].z, ra[i].w);
+            o.x = pack_bf2(ra[i].x * asc[i], ra[i].y * asc[i]);
+            o.y = pack_bf2(ra[i].z * asc[i], ra[i].w * asc[i]);
             *(uint2*)(As + (idx >> 4) * LD + (idx & 15) * 4) = o;
         }
 #pragma unroll
@@ -337,7 +371,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int gm = m0 + (mt0 + i) * 16 + (lane >> 4) * 4 + r;
-                if (gm < M) hb_epilogue<EPI>(C + (size_t)(lst ? lst[gm] : gm) * ldc + gn, acc[i][j][r], b);
+                if (gm < M) hb_epilogue<EPI>(C + (size_t)(lst ? lst[gm] : gm) * ldc + gn, acc[i][j][r], b, rm.epi_arg);
             }
         }
 }
@@ -350,6 +384,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
     __shared__ float As[BK][BM + 4];
     __shared__ float Ws[BK][64 + 4];
     __shared__ int arow[BM];
+    __shared__ float asc[BM];
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
     const int* lst = nullptr;
@@ -362,7 +397,10 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
         if (m0 >= M) return;
         lst = rm.list + (size_t)blockIdx.z * rm.cap;
     }
-    for (int r = tid; r < BM; r += 256) arow[r] = m0 + r < M ? (lst ? lst[m0 + r] : m0 + r) : -1;
+    for (int r = tid; r < BM; r += 256) {
+        arow[r] = m0 + r < M ? (lst ? lst[m0 + r] : m0 + r) : -1;
+        asc[r] = m0 + r < M && lst && rm.a_scale ? rm.a_scale[lst[m0 + r]] : 1.0f;
+    }
     __syncthreads();
     float acc[RM][4];
 #pragma unroll
@@ -373,7 +411,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
         for (int idx = tid; idx < BM * BK; idx += 256) {
             const int r = idx / BK, c = idx % BK;
             const int gm = m0 + r, gk = k0 + c;
-            As[c][r] = (gm < M && gk < K) ? A[(size_t)(lst ? arow[r] / rm.a_div : gm) * lda + gk] : 0.f;
+            As[c][r] = (gm < M && gk < K) ? A[(size_t)(lst ? arow[r] / rm.a_div : gm) * lda + gk] * asc[r] : 0.f;
         }
         for (int idx = tid; idx < 64 * BK; idx += 256) {
             const int r = idx / BK, c = idx % BK;
@@ -402,7 +440,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int gn = n0 + tx * 4 + j;
-            if (gn < N) hb_epilogue<EPI>(C + (size_t)arow[ty * RM + i] * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f);
+            if (gn < N) hb_epilogue<EPI>(C + (size_t)arow[ty * RM + i] * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f, rm.epi_arg);
         }
     }
 }
@@ -476,7 +514,7 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
 #pragma unroll
         for (int j = 0; j < HB_GEMV_CPW; ++j) {
             const float sum = hb_wave_sum(acc[m][j]);
-            if (m < M && n0 + j < N && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n0 + j, sum, bias ? bias[n0 + j] : 0.f);
+            if (m < M && n0 + j < N && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n0 + j, sum, bias ? bias[n0 + j] : 0.f, rm.epi_arg);
         }
 }
 
@@ -614,7 +652,7 @@ __global__ __launch_bounds__(512) void k_hb_gemm_rows16(const float* A, long lda
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = kb * 4 + r;
-            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((((((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col]) + red[4][row][col]) + red[5][row][col]) + red[6][row][col]) + red[7][row][col], bz);
+            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((((((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col]) + red[4][row][col]) + red[5][row][col]) + red[6][row][col]) + red[7][row][col], bz, rm.epi_arg);
         }
     }
 }
@@ -675,6 +713,7 @@ int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const
     if (epi == HB_EPI_GELU) return hb_gemm_epi<T, HB_EPI_GELU>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     if (epi == HB_EPI_TANH) return hb_gemm_epi<T, HB_EPI_TANH>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    if (epi == HB_EPI_SOFTCAP) return hb_gemm_epi<T, HB_EPI_SOFTCAP>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
 }
 
@@ -849,7 +888,184 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_mlstm_scan(const 
     if (blockIdx.z == 0 && threadIdx.x == 0) nt_[dim] = m;
 }
 
-// per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]), times
+// Rotation of the newer mixers: dims i and i + rot/2 (i < rot/2) of a vector form a pair (u, v) that position p turns by the angle
+// p * inv_freq[i] into (u cos - v sin, v cos + u sin); dims at or beyond rot pass unchanged.  x: the vector, d: the dim asked for.
+__device__ __forceinline__ float hb_rot_half(const float* x, int d, int rot, float p, const float* inv_freq) {
+    const float v = x[d];
+    if (d >= rot) return v;
+    const int half = rot >> 1, i = d < half ? d : d - half;
+    float sn, cs;
+    sincosf(p * inv_freq[i], &sn, &cs);
+    return d < half ? v * cs - x[d + half] * sn : v * cs + x[d - half] * sn;
+}
+
+// Retention: S_t = decay_h S_{t-1} + k_t v_t^T, o_t = S_t^T q_t, one fixed decay per head, no softmax and no denominator.
+// proj row = [q (H*dim) | k (H*dim) | v (H*vdim) | gate (H*vdim)].  q and k are rotated while they are staged (hb_rot_half on their
+// first `rot` dims), k is then multiplied by kscale.  Block, waves and the order of every sum as in the scans above.
+// Long portions run the request's rows in chunks of `chunk_len` side by side (modes as for the shift-decay scan below):
+//   mode 0  the whole portion from the slot's state, outputs and state stored
+//   mode 1  chunk z from a zero state, no outputs: its final state goes to the workspace
+//   mode 2  chunk z replayed from its carry (left in the workspace by k_hb_retention_carry), outputs written
+// Workspace entry of chunk k of request r: index rs / chunk_len + r + k, [H][dim*vdim] floats each.
+template <int DPW>
+__global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_retention_scan(const float* proj, long ldp, float* out, long ldo, const float* decay,
+                                                                              const float* inv_freq, float* state, const int* req_rows,
+                                                                              const int* req_state, const int* pos, int H, int dim, int vdim,
+                                                                              int rot, float kscale, int TT, int mode, int chunk_len, float* ws) {
+    extern __shared__ float sm[];
+    const int nw = blockDim.x >> 6, dpad = nw * DPW;
+    float* ks = sm;                       // [TT][dpad]
+    float* qs = ks + TT * dpad;           // [TT][dpad]
+    float* vs = qs + TT * dpad;           // [TT][64]
+    float* part = vs + TT * 64;           // [2][nw][64]
+    const int vt = (vdim + 63) >> 6, chunk = mode == 0 ? 0 : blockIdx.z / vt, tile = mode == 0 ? blockIdx.z : blockIdx.z % vt;
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = tile * 64 + lane;
+    const int d0 = w * DPW;
+    const int rs0 = req_rows[r], re0 = req_rows[r + 1];
+    const int rs = mode == 0 ? rs0 : rs0 + chunk * chunk_len;
+    if (rs >= re0) return;
+    const int re = mode == 0 || rs + chunk_len > re0 ? re0 : rs + chunk_len;
+    const bool ok = c < vdim, fresh = pos[rs0] == 0;
+    float* St = state + ((size_t)req_state[r] * H + h) * dim * vdim;
+    if (mode != 0) St = ws + ((size_t)(rs0 / chunk_len + r + chunk) * H + h) * ((size_t)dim * vdim);
+    const bool load = mode == 2 || (mode == 0 && !fresh);
+    const float dec = decay[h];
+    float S[DPW];
+#pragma unroll
+    for (int i = 0; i < DPW; ++i) S[i] = (ok && load && d0 + i < dim) ? St[(size_t)(d0 + i) * vdim + c] : 0.f;
+    int flip = 0;
+    for (int t0 = rs; t0 < re; t0 += TT) {
+        const int nt = re - t0 < TT ? re - t0 : TT;
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nt * dpad; idx += blockDim.x) {
+            const int tt = idx / dpad, d = idx - tt * dpad;
+            float q = 0.f, k = 0.f;
+            if (d < dim) {
+                const float* p = proj + (size_t)(t0 + tt) * ldp + h * dim;
+                const float pf = (float)pos[t0 + tt];
+                k = hb_rot_half(p + H * dim, d, rot, pf, inv_freq) * kscale;
+                if (mode != 1) q = hb_rot_half(p, d, rot, pf, inv_freq);
+            }
+            qs[idx] = q;
+            ks[idx] = k;
+        }
+        for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
+            const int tt = idx >> 6, cc = tile * 64 + (idx & 63);
+            vs[idx] = cc < vdim ? proj[(size_t)(t0 + tt) * ldp + 2 * H * dim + h * vdim + cc] : 0.f;
+        }
+        __syncthreads();
+        if (mode == 1) {
+            for (int tt = 0; tt < nt; ++tt) {
+                const float v = vs[tt * 64 + lane];
+                const float* kt = ks + tt * dpad + d0;
+#pragma unroll
+                for (int i = 0; i < DPW; ++i) S[i] = dec * S[i] + kt[i] * v;
+            }
+            continue;
+        }
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = vs[tt * 64 + lane];
+            const float* kt = ks + tt * dpad + d0;
+            const float* qt = qs + tt * dpad + d0;
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < DPW; ++i) {
+                const float sv = dec * S[i] + kt[i] * v;
+                S[i] = sv;
+                o = fmaf(sv, qt[i], o);
+            }
+            float* pt = part + flip * nw * 64;
+            pt[w * 64 + lane] = o;
+            __syncthreads();
+            if (w == 0 && ok) {
+                float sum = pt[lane];
+                for (int k2 = 1; k2 < nw; ++k2) sum += pt[k2 * 64 + lane];
+                out[(size_t)(t0 + tt) * ldo + h * vdim + c] = sum;
+            }
+            flip ^= 1;
+        }
+    }
+    if (mode == 2) return;
+    if (ok)
+#pragma unroll
+        for (int i = 0; i < DPW; ++i)
+            if (d0 + i < dim) St[(size_t)(d0 + i) * vdim + c] = S[i];
+}
+// Between the two chunked passes: the slot's state is pushed through the request's chunks in order, S <- decay^rows S + B_k; every
+// chunk's workspace entry receives its carry-in in place of B_k, the slot the final state.  decay^rows is formed by repeated
+// multiplication (at most chunk_len factors).
+__global__ __launch_bounds__(256) void k_hb_retention_carry(float* ws, float* state, const float* decay, const int* req_rows, const int* req_state,
+                                                            const int* pos, int H, int dim, int vdim, int chunk_len) {
+    const int r = blockIdx.x, h = blockIdx.y;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const int nc = (re - rs + chunk_len - 1) / chunk_len;
+    const bool fresh = pos[rs] == 0;
+    const size_t per = (size_t)dim * vdim;
+    float* St = state + ((size_t)req_state[r] * H + h) * per;
+    float* w0 = ws + ((size_t)(rs / chunk_len + r) * H + h) * per;
+    const float dec = decay[h];
+    float full = 1.f, last = 1.f;
+    for (int i = 0; i < chunk_len; ++i) full *= dec;
+    for (int i = 0; i < (re - rs) - (nc - 1) * chunk_len; ++i) last *= dec;
+    for (size_t e = (size_t)blockIdx.z * 256 + threadIdx.x; e < per; e += (size_t)256 * gridDim.z) {
+        float S = fresh ? 0.f : St[e];
+        for (int k = 0; k < nc; ++k) {
+            float* wk = w0 + (size_t)k * H * per;
+            const float B = wk[e];
+            wk[e] = S;
+            S = (k == nc - 1 ? last : full) * S + B;
+        }
+        St[e] = S;
+    }
+}
+
+// ---- latent attention: what a row leaves in the cache, and its query ----------------------------------------------------------
+// sum of v over a block of 256 threads in a fixed order: butterfly per wave, the four wave sums added in wave order
+__device__ __forceinline__ float hb_block_sum256(float v, float* red) {
+    v = hb_wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return ((red[0] + red[1]) + red[2]) + red[3];
+}
+// proj row = [query latent (q_rank) | key / value latent (R) | rotated key part (r) | gate (H) | ...].  Block (row, 0): the query latent
+// is RMS-normed with its weight in place.  Block (row, 1): the key / value latent is RMS-normed with its weight into the row's cache
+// entry [R + r] (engine dtype), followed by the rotated key part (hb_rot_half on its first `rot` dims).
+template <typename T>
+__global__ __launch_bounds__(256) void k_hb_latent_prep(float* proj, long ldp, T* cache, const float* qn, const float* kn, const float* inv_freq,
+                                                        const int* pos, const int* page, const int* slot, int q_rank, int R, int r, int rot,
+                                                        int ps, float eps) {
+    __shared__ float red[4];
+    const int row = blockIdx.x;
+    float* p = proj + (size_t)row * ldp;
+    if (blockIdx.y == 0) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < q_rank; i += 256) ss = fmaf(p[i], p[i], ss);
+        const float inv = 1.0f / sqrtf(hb_block_sum256(ss, red) / (float)q_rank + eps);
+        for (int i = threadIdx.x; i < q_rank; i += 256) p[i] = p[i] * inv * qn[i];
+        return;
+    }
+    const float* x = p + q_rank;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < R; i += 256) ss = fmaf(x[i], x[i], ss);
+    const float inv = 1.0f / sqrtf(hb_block_sum256(ss, red) / (float)R + eps);
+    T* dst = cache + ((size_t)page[row] * ps + slot[row]) * (size_t)(R + r);
+    for (int i = threadIdx.x; i < R; i += 256) hb_st(dst + i, x[i] * inv * kn[i]);
+    const float pf = (float)pos[row];
+    for (int d = threadIdx.x; d < r; d += 256) hb_st(dst + R + d, hb_rot_half(x + R, d, rot, pf, inv_freq));
+}
+// q row = per head [plain (dim) | rotated (r)]; qa row = per head [query against the latent (R) | rotated part (r)].  The first part
+// of qa is a product of its own (the plain part times the head's key expansion); this fills the second.
+__global__ __launch_bounds__(64) void k_hb_latent_qrot(const float* q, long ldq, float* qa, long ldqa, const float* inv_freq, const int* pos, int dim,
+                                                       int R, int r, int rot) {
+    const int row = blockIdx.x, h = blockIdx.y;
+    const float* src = q + (size_t)row * ldq + (size_t)h * (dim + r) + dim;
+    float* dst = qa + (size_t)row * ldqa + (size_t)h * (R + r) + R;
+    const float pf = (float)pos[row];
+    for (int d = threadIdx.x; d < r; d += 64) dst[d] = hb_rot_half(src, d, rot, pf, inv_freq);
+}
+
+// per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]; NULL: none), times
 // a gate (gate_mode 1: sigmoid(g), 2: g * sigmoid(g); g = proj[row][gate_off + h*vdim + j]), times out_scale.  In place.
 enum { HB_GATE_NONE = 0, HB_GATE_SIGMOID = 1, HB_GATE_SILU = 2 };
 __global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const float* w, int per_head_w, const float* proj, long ldp, int gate_off,
@@ -861,7 +1077,8 @@ __global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const f
     ss = hb_wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
     for (int j = lane; j < vdim; j += 64) {
-        float v = p[j] * inv * w[per_head_w ? h * vdim + j : j];
+        float v = p[j] * inv;
+        if (w) v *= w[per_head_w ? h * vdim + j : j];
         if (gate_mode != HB_GATE_NONE) {
             const float g = proj[(size_t)row * ldp + gate_off + h * vdim + j];
             v *= gate_mode == HB_GATE_SIGMOID ? hb_sigmoid(g) : g * hb_sigmoid(g);
@@ -1415,7 +1632,8 @@ __device__ __forceinline__ float hb_dot_slices(const float* q, const bf16_t* k, 
 template <typename T>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
-                          long v_base, float scale, int split, int seg_chunks, float* part, int gated, float out_scale) {
+                          long v_base, float scale, int split, int seg_chunks, float* part, const float* gate, long ldg, float out_scale,
+                          int Gc, long v_ld) {
     extern __shared__ float sm[];
     const int QG = H / G, NWV = QG * split;
     const int dimp = (dim + 3) & ~3;
@@ -1425,6 +1643,10 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
     float* mo = qs + QG * dimp;             // [NWV][vdim + 2]: partial output, maximum, sum of each wave
     const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int qh = wv % QG, sp = wv / QG, hq = g * QG + qh;
+    // Gc heads per cached row (Gc = G: one per block row of the grid; Gc = 1 < G: every group of query heads reads the one shared head),
+    // value rows v_ld apart
+    const int gk = g % Gc;
+    const size_t kld = (size_t)Gc * dim;
     const int p = pos[row];
     const int* pt = ptab + (size_t)row_req[row] * pts;
     const int first = p - window + 1;
@@ -1475,7 +1697,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
             // a chunk of cached tokens only, one 128-dim slice: all sixteen row requests of the wave go out before the first is used
             const int sub = lane & 15, grp = lane >> 4;
             const bool mine_ok = sub * 8 < dim;
-            const bf16_t* kb = (const bf16_t*)cache + g * dim + (mine_ok ? sub * 8 : 0);
+            const bf16_t* kb = (const bf16_t*)cache + gk * dim + (mine_ok ? sub * 8 : 0);
             float4 qa = make_float4(0.f, 0.f, 0.f, 0.f), qb = qa;
             if (mine_ok) { qa = *(const float4*)(q + sub * 8); qb = *(const float4*)(q + sub * 8 + 4); }
 #pragma unroll
@@ -1485,7 +1707,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
                 for (int i8 = 0; i8 < 8; ++i8) {
                     const int it = half * 8 + i8;
                     const int kk = it * 4 + grp < cnt ? it * 4 + grp : cnt - 1;
-                    kreg[i8] = *(const uint4*)(kb + (size_t)wloc[kk] * (size_t)(G * dim));
+                    kreg[i8] = *(const uint4*)(kb + (size_t)wloc[kk] * kld);
                 }
 #pragma unroll
                 for (int i8 = 0; i8 < 8; ++i8) {
@@ -1519,7 +1741,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
                         part = fmaf(b2.x, k1.x, part); part = fmaf(b2.y, k1.y, part); part = fmaf(b2.z, k1.z, part); part = fmaf(b2.w, k1.w, part);
                     }
                 } else {
-                    part = hb_dot_slices(q, cache + (size_t)w * (size_t)(G * dim) + g * dim, dim, sub);
+                    part = hb_dot_slices(q, cache + (size_t)w * kld + gk * dim, dim, sub);
                 }
                 part += __shfl_xor(part, 8, 64);
                 part += __shfl_xor(part, 4, 64);
@@ -1530,7 +1752,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
             }
         } else if (u < total) {
             dot = where < 0 ? hb_dot_row(q, pool + (size_t)(-where - 1) * pw, dim, pvec)
-                            : hb_dot_row(q, cache + (size_t)where * (size_t)(G * dim) + g * dim, dim, kvec);
+                            : hb_dot_row(q, cache + (size_t)where * kld + gk * dim, dim, kvec);
         }
         const float sc = u < total ? dot * scale : -INFINITY;
         const float mn = fmaxf(m, hb_wave_max(sc));
@@ -1545,7 +1767,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
         // acc[e] belongs to value column hb_vcol(e): with a bf16 cache and an even vdim a lane owns two adjacent columns of each
         // 128-column group (one 4-byte request per key), else one column of each 64-column group.
         const int npool = nb - base < 0 ? 0 : (nb - base < cnt ? nb - base : cnt);
-        const size_t gv = (size_t)G * vdim;
+        const size_t gv = (size_t)v_ld;
         if (pair) {
 #pragma unroll
             for (int c = 0; c < HB_MAX_VPL / 2; ++c) {
@@ -1553,7 +1775,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
                     const int j = c * 128 + 2 * lane;
                     const int jj = j < vdim ? j : vdim - 2;
                     const float* pbase = pool + dim + jj;
-                    const T* vbase = cache + v_base + g * vdim + jj;
+                    const T* vbase = cache + v_base + gk * vdim + jj;
                     float a0 = acc[2 * c] * alpha, a1 = acc[2 * c + 1] * alpha;
                     for (int k0 = 0; k0 < npool; k0 += 8) {
                         float pv[8];
@@ -1590,7 +1812,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
             if (c * 64 < vdim) {
                 const int jj = j < vdim ? j : vdim - 1;
                 const float* pbase = pool + dim + jj;
-                const T* vbase = cache + v_base + g * vdim + jj;
+                const T* vbase = cache + v_base + gk * vdim + jj;
                 float a = acc[c] * alpha;
                 for (int k0 = 0; k0 < npool; k0 += 8) {
                     float pv[8], vv[8];
@@ -1650,22 +1872,21 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
             if (lane == 0) { dst[vdim] = mm; dst[vdim + 1] = lt; }
             return;
         }
-        const float gate = (gated ? hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]) : 1.0f) * out_scale;
+        const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
         for (int j = lane; j < vdim; j += 64) {
             float a = 0.f;
             for (int s2 = 0; s2 < split; ++s2) {
                 const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
                 a += o2[j] * expf(o2[vdim] - mm);
             }
-            out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
+            out[(size_t)row * ldo + hq * vdim + j] = a / lt * gmul;
         }
     }
 }
 
 // few-row steps: the segments' partial results of a (row, head), merged in segment order; output gate applied here
-__global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, const float* proj, long ldp, float* out, long ldo,
-                                                      const int* pos, int H, int G, int dim, int vdim, int window, int P, int seg_chunks, int gated,
-                                                      float out_scale) {
+__global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, float* out, long ldo, const int* pos, int H, int vdim,
+                                                      int window, int P, int seg_chunks, const float* gate, long ldg, float out_scale) {
     const int row = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
     const int p = pos[row];
     const int first = p - window + 1;
@@ -1676,11 +1897,11 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
     for (int s2 = 0; s2 < nseg; ++s2) mm = fmaxf(mm, src[(size_t)s2 * (vdim + 2) + vdim]);
     float lt = 0.f;
     for (int s2 = 0; s2 < nseg; ++s2) lt += src[(size_t)s2 * (vdim + 2) + vdim + 1] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
-    const float gate = (gated ? hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]) : 1.0f) * out_scale;
+    const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
     for (int j = lane; j < vdim; j += 64) {
         float a = 0.f;
         for (int s2 = 0; s2 < nseg; ++s2) a += src[(size_t)s2 * (vdim + 2) + j] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
-        out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
+        out[(size_t)row * ldo + hq * vdim + j] = a / lt * gmul;
     }
 }
 
@@ -1688,8 +1909,9 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
 // One block per row: router logits z_j = router[j] . h in fp32 (lane-strided sums over four waves and a butterfly: an order fixed by
 // the width, the same for every step shape), then one wave: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
 // index wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
+// sigmoid != 0: s_j = sigmoid(z_j) instead of the softmax; renorm == 0: the weights are the chosen s as they are.
 __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh, const float* router, const float* corr, int W, int nE, int top,
-                                                       int* sel, float* wgt) {
+                                                       int* sel, float* wgt, int sigmoid, int renorm) {
     extern __shared__ float sm[];
     float* sc = sm;                    // [nE] logits, then scores
     float* ch = sm + nE;               // [nE] choice values
@@ -1751,20 +1973,28 @@ __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh,
     for (int i = lane; i < nE; i += 64) sc[i] = ((part[i] + part[nE + i]) + part[2 * nE + i]) + part[3 * nE + i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
-    float mx = -INFINITY;
-    for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, sc[i]);
-    mx = hb_wave_max(mx);
-    float sum = 0.f;
-    for (int i = lane; i < nE; i += 64) {
-        const float e = expf(sc[i] - mx);
-        sc[i] = e;
-        sum += e;
-    }
-    sum = hb_wave_sum(sum);
-    for (int i = lane; i < nE; i += 64) {
-        const float v = sc[i] / sum;
-        sc[i] = v;
-        ch[i] = v + (corr ? corr[i] : 0.f);
+    if (sigmoid) {
+        for (int i = lane; i < nE; i += 64) {
+            const float v = hb_sigmoid(sc[i]);
+            sc[i] = v;
+            ch[i] = v + (corr ? corr[i] : 0.f);
+        }
+    } else {
+        float mx = -INFINITY;
+        for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, sc[i]);
+        mx = hb_wave_max(mx);
+        float sum = 0.f;
+        for (int i = lane; i < nE; i += 64) {
+            const float e = expf(sc[i] - mx);
+            sc[i] = e;
+            sum += e;
+        }
+        sum = hb_wave_sum(sum);
+        for (int i = lane; i < nE; i += 64) {
+            const float v = sc[i] / sum;
+            sc[i] = v;
+            ch[i] = v + (corr ? corr[i] : 0.f);
+        }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
@@ -1795,7 +2025,7 @@ __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh,
     const float den = wsum + 1e-20f;
     for (int k = lane; k < top; k += 64) {
         sel[(size_t)row * top + k] = pick[k];
-        wgt[(size_t)row * top + k] = sc[pick[k]] / den;
+        wgt[(size_t)row * top + k] = renorm ? sc[pick[k]] / den : sc[pick[k]];
     }
 }
 // Block e lists the entries (row*top + k) routed to expert e, ascending: list[e*cap + 0 .. count[e]).
@@ -1821,23 +2051,27 @@ __global__ __launch_bounds__(256) void k_hb_moe_group(const int* sel, int n_entr
     }
     if (threadIdx.x == 0) count[e] = base;
 }
-// y = g * sigmoid(alpha g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gu row = [gate (ff) | up (ff)].
+// y = act(g) * (u + up_offset), g = min(gate, limit), u = clamp(up, -limit, limit); act(g) = g * sigmoid(alpha g), or the tanh form
+// of gelu (gelu != 0); gu row = [gate (ff) | up (ff)].
 // sel != NULL: rows are routed entries, those of identity outputs (sel >= experts) are skipped.
-__global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y, int ff, float limit, float alpha, const int* sel, int experts) {
+__device__ __forceinline__ float hb_glu(float g0, float u0, float limit, float alpha, float up_offset, int gelu) {
+    const float g = fminf(g0, limit), u = fminf(fmaxf(u0, -limit), limit);
+    return (gelu ? hb_gelu_tanh(g) : g * hb_sigmoid(alpha * g)) * (u + up_offset);
+}
+__global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y, int ff, float limit, float alpha, const int* sel, int experts,
+                                                      float up_offset, int gelu) {
     const int row = blockIdx.x;
     if (sel && sel[row] >= experts) return;
-    for (int j = blockIdx.y * 256 + threadIdx.x; j < ff; j += gridDim.y * 256) {
-        const float g = fminf(gu[(size_t)row * 2 * ff + j], limit);
-        const float u = fminf(fmaxf(gu[(size_t)row * 2 * ff + ff + j], -limit), limit);
-        y[(size_t)row * ff + j] = g * hb_sigmoid(alpha * g) * (u + 1.0f);
-    }
+    for (int j = blockIdx.y * 256 + threadIdx.x; j < ff; j += gridDim.y * 256)
+        y[(size_t)row * ff + j] = hb_glu(gu[(size_t)row * 2 * ff + j], gu[(size_t)row * 2 * ff + ff + j], limit, alpha, up_offset, gelu);
 }
 // Few-row steps.  Entries per row: its `top` routed choices, then (shared_ff > 0) the shared expert.
 struct hb_moe_small {
     const int* sel;
     const float* wgt;
     int top, experts, ff, shared_ff, ld_act;
-    float limit, shared_limit, alpha;
+    float limit, shared_limit, alpha, up_offset;
+    int scale_input;        // the routing weight multiplies the expert's input instead of its output
 };
 // gate / up products + activation of every entry: block (column tile, entry); a wave takes gate row n and up row ff + n of the
 // entry's expert and stores g * sigmoid(alpha g) * (u + 1) with the clamps of that expert.  act row of an entry: ld_act floats.
@@ -1848,13 +2082,14 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
     const int entry = blockIdx.y, row = entry / per, slot = entry - row * per, lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
     const T* wg;
     int N;
-    float limit;
+    float limit, xs = 1.0f;
     if (slot < q.top) {
         const int e = q.sel[(size_t)row * q.top + slot];
         if (e >= q.experts) return;
         wg = w_gate_up + (size_t)e * 2 * q.ff * W;
         N = q.ff;
         limit = q.limit;
+        if (q.scale_input) xs = q.wgt[(size_t)row * q.top + slot];
     } else {
         wg = shared_gate_up;
         N = q.shared_ff;
@@ -1864,11 +2099,8 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     const float* x = h + (size_t)row * ldh;
     const bool vec = (W % CH == 0) && ((((size_t)wg) & 15) == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0);
-    const float g0 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane), u0 = hb_dot_wave<T>(wg + (size_t)(N + n) * W, x, W, vec, lane);
-    if (lane == 0) {
-        const float g = fminf(g0, limit), u = fminf(fmaxf(u0, -limit), limit);
-        act[(size_t)entry * q.ld_act + n] = g * hb_sigmoid(q.alpha * g) * (u + 1.0f);
-    }
+    const float g0 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane, xs), u0 = hb_dot_wave<T>(wg + (size_t)(N + n) * W, x, W, vec, lane, xs);
+    if (lane == 0) act[(size_t)entry * q.ld_act + n] = hb_glu(g0, u0, limit, q.alpha, q.up_offset, 0);
 }
 // down products of a row's entries, weighted and added to the residual stream: a wave per (row, output column):
 // x[row][c] += sum_k wgt_k * (identity ? h[row][c] : down_{e_k}[c] . act_k)  +  shared_down[c] . act_shared, k ascending.
@@ -1883,8 +2115,9 @@ __global__ __launch_bounds__(256) void k_hb_moe_down_combine(const float* h, lon
     float acc = 0.f;
     for (int k = 0; k < q.top; ++k) {
         const int e = q.sel[(size_t)row * q.top + k];
-        const float wk = q.wgt[(size_t)row * q.top + k];
-        if (e >= q.experts) { acc = fmaf(wk, h[(size_t)row * ldh + c], acc); continue; }
+        const float wk0 = q.wgt[(size_t)row * q.top + k];
+        if (e >= q.experts) { acc = fmaf(wk0, h[(size_t)row * ldh + c], acc); continue; }
+        const float wk = q.scale_input ? 1.0f : wk0;
         const T* wd = w_down + ((size_t)e * W + c) * q.ff;
         const bool vec = avec && (q.ff % CH == 0) && ((((size_t)w_down) & 15) == 0);
         acc = fmaf(wk, hb_dot_wave<T>(wd, act + (size_t)(row * per + k) * q.ld_act, q.ff, vec, lane), acc);
@@ -1896,14 +2129,16 @@ __global__ __launch_bounds__(256) void k_hb_moe_down_combine(const float* h, lon
     if (lane == 0) x[(size_t)row * ldx + c] += acc;
 }
 // x[row] += sum_k wgt[row*top + k] * (identity output ? h[row] : expert_out[row*top + k]), k ascending
+// (scale_input: an expert's output enters with weight 1, its input was scaled instead)
 __global__ __launch_bounds__(256) void k_hb_moe_combine(float* x, long ldx, const float* h, long ldh, const float* eo, const int* sel,
-                                                        const float* wgt, int top, int experts, int W) {
+                                                        const float* wgt, int top, int experts, int W, int scale_input) {
     const int row = blockIdx.x;
     for (int i = threadIdx.x; i < W; i += 256) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k) {
             const size_t en = (size_t)row * top + k;
-            acc = fmaf(wgt[en], sel[en] >= experts ? h[(size_t)row * ldh + i] : eo[en * W + i], acc);
+            const bool ident = sel[en] >= experts;
+            acc = fmaf(scale_input && !ident ? 1.0f : wgt[en], ident ? h[(size_t)row * ldh + i] : eo[en * W + i], acc);
         }
         x[(size_t)row * ldx + i] += acc;
     }
@@ -1963,6 +2198,8 @@ struct vox_hybrid {
     std::vector<vox_hybrid_run> runs;
     vox_hybrid_weights w;
     float *xa = nullptr, *xb = nullptr, *h = nullptr, *h2 = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
+    float *ff_act = nullptr;                // [max_rows][max gated dense width]: activation output of the gated dense feed-forward
+    int max_gated = 0;
     float *shift = nullptr;                 // [5][max_rows][width]: token-shift mixes
     float *scan_ws = nullptr;               // chunk states and decay products of the chunked matrix-state scan
     size_t scan_ws_floats = 0;
@@ -1974,9 +2211,32 @@ struct vox_hybrid {
     int max_in = 0, max_mix = 0, max_ff = 0;
     int max_ne = 0, max_top = 0, max_eff = 0, max_experts = 0;
     bool any_shift = false;
+    bool attn_big_lds = false;              // the attention kernel was given the right to more than 64 KB of LDS
 };
 
-static bool hb_is_attn(int kind) { return kind == VOX_MIXER_POOLED_WINDOW_ATTN || kind == VOX_MIXER_CAUSAL_ATTN; }
+static bool hb_is_attn(int kind) { return kind == VOX_MIXER_POOLED_WINDOW_ATTN || kind == VOX_MIXER_CAUSAL_ATTN || kind == VOX_MIXER_LATENT_ATTN; }
+static inline int hb_up4(int v) { return (v + 3) & ~3; }
+// Where a latent-attention row keeps what it derives from the fused projection [query latent | kv latent | rotated key | gate]:
+// q = per head [plain | rotated] at off_q, the query against the cached rows (per head [R | r]) at off_qa, the weighted sum of cached
+// latents per head at off_o.  Every part starts on a 16-byte boundary.
+struct hb_latent_layout {
+    int n_in, off_q, off_qa, off_o, n_proj;
+};
+static hb_latent_layout hb_latent(const vox_hybrid_layer& L) {
+    hb_latent_layout y;
+    y.n_in = L.q_rank + L.kv_rank + L.rot_dim + L.heads;
+    y.off_q = hb_up4(y.n_in);
+    y.off_qa = y.off_q + hb_up4(L.heads * (L.dim + L.rot_dim));
+    y.off_o = y.off_qa + hb_up4(L.heads * (L.kv_rank + L.rot_dim));
+    y.n_proj = y.off_o + hb_up4(L.heads * L.kv_rank);
+    return y;
+}
+// query heads per block of the latent attention: all heads read the one cached row; at most 16 share a block
+static int hb_latent_groups(int H) {
+    for (int g = 1; g <= H; ++g)
+        if (H % g == 0 && H / g <= 16) return g;
+    return H;
+}
 // rows of the fused input projection
 static int hb_layer_in(const vox_hybrid_layer& L) {
     switch (L.kind) {
@@ -1986,6 +2246,8 @@ static int hb_layer_in(const vox_hybrid_layer& L) {
         case VOX_MIXER_RGLRU: return 2 * L.heads * L.dim;
         case VOX_MIXER_CAUSAL_ATTN: return L.heads * L.dim + L.kv_heads * (L.dim + L.vdim);
         case VOX_MIXER_SHIFT_DECAY: return 4 * L.heads * L.dim + L.lora;
+        case VOX_MIXER_LATENT_ATTN: return L.q_rank + L.kv_rank + L.rot_dim + L.heads;
+        case VOX_MIXER_RETENTION: return 2 * L.heads * L.dim + 2 * L.heads * L.vdim;
     }
     return -1;
 }
@@ -1993,6 +2255,7 @@ static int hb_layer_in(const vox_hybrid_layer& L) {
 static int hb_layer_proj(const vox_hybrid_layer& L) {
     if (L.kind == VOX_MIXER_RGLRU) return 5 * L.heads * L.dim;                           // + conv output, 2 gates
     if (L.kind == VOX_MIXER_SHIFT_DECAY) return 5 * L.heads * L.dim + L.lora;            // + decay pre-activation
+    if (L.kind == VOX_MIXER_LATENT_ATTN) return hb_latent(L).n_proj;
     return hb_layer_in(L);
 }
 
@@ -2104,6 +2367,68 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
                            io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap, tt);
         hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj,
                            2 * L.heads * L.dim + L.heads * L.vdim, (int)HB_GATE_SIGMOID, L.vdim, c.eps, L.out_scale);
+    } else if (L.kind == VOX_MIXER_RETENTION) {
+        auto kern = dpw == 16 ? k_hb_retention_scan<16> : (dpw == 32 ? k_hb_retention_scan<32> : k_hb_retention_scan<64>);
+        const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
+        const float kscale = 1.0f / sqrtf((float)L.dim);
+        if (n > HB_SCAN_CHUNK && m->scan_ws) {
+            // steps of many rows: chunks of HB_SCAN_CHUNK rows side by side (reduce from zero, carries in order, replay)
+            const int nch = (n + HB_SCAN_CHUNK - 1) / HB_SCAN_CHUNK;
+            const int per = L.dim * L.vdim;
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.decay,
+                               L.inv_freq, state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.rot_dims, kscale, tt, 1,
+                               HB_SCAN_CHUNK, m->scan_ws);
+            hipLaunchKernelGGL(k_hb_retention_carry, dim3(n_req, L.heads, (per + 255) / 256 < 64 ? (per + 255) / 256 : 64), dim3(256), 0, st,
+                               m->scan_ws, state, L.decay, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, HB_SCAN_CHUNK);
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.decay,
+                               L.inv_freq, state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.rot_dims, kscale, tt, 2,
+                               HB_SCAN_CHUNK, m->scan_ws);
+        } else {
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.decay,
+                               L.inv_freq, state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.rot_dims, kscale, tt, 0, 0,
+                               (float*)nullptr);
+        }
+        hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj,
+                           2 * L.heads * L.dim + L.heads * L.vdim, (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
+    } else if (L.kind == VOX_MIXER_LATENT_ATTN) {
+        const hb_latent_layout y = hb_latent(L);
+        const int H = L.heads, R = L.kv_rank, r = L.rot_dim, D = R + r, dq = L.dim + r;
+        float* q = m->proj + y.off_q;
+        float* qa = m->proj + y.off_qa;
+        float* o = m->proj + y.off_o;
+        hipLaunchKernelGGL((k_hb_latent_prep<T>), dim3(n, 2), dim3(256), 0, st, m->proj, (long)n_proj, (T*)cache, L.q_lat_norm, L.kv_lat_norm,
+                           L.inv_freq, io->pos, io->page, io->slot, L.q_rank, R, r, L.rot_dims, ps, c.eps);
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj, n_proj, (const T*)L.w_uq, nullptr, q, n_proj, n, H * dq, L.q_rank));
+        // every head's plain query part times its key expansion: the query against the cached latent
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, q, n_proj, (const T*)L.w_ukT, nullptr, qa, n_proj, n, R, L.dim,
+                           hb_rowmap{nullptr, nullptr, 0, 1, (long)R * L.dim, (long)dq, (long)D, 0, nullptr, 0.f}, H));
+        if (r > 0)
+            hipLaunchKernelGGL(k_hb_latent_qrot, dim3(n, H), dim3(64), 0, st, q, (long)n_proj, qa, (long)n_proj, L.inv_freq, io->pos, L.dim, R, r,
+                               L.rot_dims);
+        // attention of all heads over one cached head of D key dims whose first R dims are also the value
+        const int G = hb_latent_groups(H), QG = H / G;
+        const int window = L.window > 0 ? L.window : c.max_seq_len, P = 0x7fffffff;
+        const int split = 16 / QG >= 4 ? 4 : (16 / QG >= 1 ? 16 / QG : 1);
+        const int nwv2 = QG * split, dimp = (D + 3) & ~3;
+        const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (R + 2) * 4;
+        const int max_keys = max_kvlen < window ? max_kvlen : window;
+        const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+        const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (R + 2) * 4 <= m->attn_ws_bytes;
+        const float* gate = m->proj + L.q_rank + D;
+        if (lds > 64 * 1024 && !m->attn_big_lds) {
+            VOX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_hb_attn<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            m->attn_big_lds = true;
+        }
+        hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, qa, (long)n_proj, (const T*)cache,
+                           (const float*)nullptr, o, (long)n_proj, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, D, R, window, P, ps, 1,
+                           0L, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr, gate, (long)n_proj,
+                           L.out_scale, 1, (long)D);
+        if (segmented)
+            hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, o, (long)n_proj, io->pos, H, R, window, P,
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale);
+        // every head's weighted latent times its value expansion
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, o, n_proj, (const T*)L.w_uv, nullptr, m->mix, n_mix, n, L.vdim, R,
+                           hb_rowmap{nullptr, nullptr, 0, 1, (long)L.vdim * R, (long)R, (long)L.vdim, 0, nullptr, 0.f}, H));
     } else if (L.kind == VOX_MIXER_RGLRU) {
         const int C = L.heads * L.dim, bs = L.dim;
         hipLaunchKernelGGL(k_hb_conv_causal, dim3(n, (C + 255) / 256), dim3(256), 0, st, m->proj, (long)n_proj, L.conv_w, L.conv_b, state, io->pos,
@@ -2142,13 +2467,14 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         const int max_keys = causal ? max_kvlen : (max_kvlen < window ? max_kvlen : window) + max_kvlen / P + 1;
         const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
         const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (L.vdim + 2) * 4 <= m->attn_ws_bytes;
+        const float* gate = causal ? (const float*)nullptr : m->proj + H * L.dim + G * L.dim + G * L.vdim;      // one logit per query head
         hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, m->proj, (long)n_proj, (const T*)cache,
                            pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, window,
                            P, ps, ppp, v_base, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr,
-                           causal ? 0 : 1, L.out_scale);
+                           gate, (long)n_proj, L.out_scale, G, (long)G * L.vdim);
         if (segmented)
-            hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->proj, (long)n_proj, m->mix, (long)n_mix,
-                               io->pos, H, G, L.dim, L.vdim, window, P, HB_ATTN_SEG, causal ? 0 : 1, L.out_scale);
+            hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->mix, (long)n_mix, io->pos, H, L.vdim, window, P,
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale);
     }
     return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
 }
@@ -2159,10 +2485,11 @@ template <typename T>
 static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n) {
     const int W = m->cfg.width, nE = E.experts + E.identity, top = E.top, ne = n * top, ff = E.ff;
     hipLaunchKernelGGL(k_hb_moe_router, dim3(n), dim3(256), (size_t)(6 * nE + top) * 4, st, h2, (long)W, E.router, E.correction, W, nE, top,
-                       m->moe_sel, m->moe_wgt);
+                       m->moe_sel, m->moe_wgt, E.score_kind == VOX_ROUTER_SIGMOID ? 1 : 0, E.renorm);
     if (n <= HB_MOE_GEMV_ROWS) {
         const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;
-        const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha};
+        const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha, E.up_offset,
+                             E.scale_input};
         if (maxf > 0 && per > 0 && (E.experts > 0 || E.shared_ff > 0))
             hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
                                (const T*)E.shared_gate_up, m->moe_act, W, q);
@@ -2174,18 +2501,20 @@ static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const 
         const int cap = m->cfg.max_rows;
         hipLaunchKernelGGL(k_hb_moe_group, dim3(E.experts), dim3(256), 0, st, m->moe_sel, ne, cap, m->moe_list, m->moe_count);
         VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)2 * ff, n, 2 * ff, W,
-                                            hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W, 0, 0, 0}, E.experts));
+                                            hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W, 0, 0, 0,
+                                                      E.scale_input ? m->moe_wgt : (const float*)nullptr, 0.f}, E.experts));
         hipLaunchKernelGGL(k_hb_glu_clamp, dim3(ne, (ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, ff, E.limit, E.act_alpha,
-                           m->moe_sel, E.experts);
+                           m->moe_sel, E.experts, E.up_offset, 0);
         VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, m->moe_act, (long)ff, (const T*)E.w_down, nullptr, m->moe_out, (long)W, n, W, ff,
                                             hb_rowmap{m->moe_count, m->moe_list, cap, 1, (long)W * ff, 0, 0, 0}, E.experts));
     }
-    hipLaunchKernelGGL(k_hb_moe_combine, dim3(n), dim3(256), 0, st, cur, ldx, h2, (long)W, m->moe_out, m->moe_sel, m->moe_wgt, top, E.experts, W);
+    hipLaunchKernelGGL(k_hb_moe_combine, dim3(n), dim3(256), 0, st, cur, ldx, h2, (long)W, m->moe_out, m->moe_sel, m->moe_wgt, top, E.experts, W,
+                       E.scale_input);
     if (E.shared_ff > 0) {
         const int sf = E.shared_ff;
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, h2, W, (const T*)E.shared_gate_up, nullptr, m->ff, 2 * sf, n, 2 * sf, W));
         hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (sf + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, sf, E.shared_limit, E.act_alpha,
-                           (const int*)nullptr, 0);
+                           (const int*)nullptr, 0, E.up_offset, 0);
         VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->moe_act, sf, (const T*)E.shared_down, nullptr, cur, ldx, n, W, sf));
     }
     return VOX_OK;
@@ -2196,7 +2525,12 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
     const vox_hybrid_config& c = m->cfg;
     const int W = c.width;
     const long ldx = 2L * W;
-    hipLaunchKernelGGL((k_hb_embed<T>), dim3(n), dim3(256), 0, st, (const T*)m->w.embedding, ids, 1, m->xa, m->xb, W, c.vocab, c.embed_scale);
+    const bool bigram = c.bigram_buckets > 0 && m->w.bigram && m->w.prev_token;
+    const hb_bigram bg{bigram ? m->w.bigram : nullptr, m->w.prev_token, c.bigram_buckets, c.bigram_mul_prev, c.bigram_mul_cur, n == n_req ? 1 : 0};
+    hipLaunchKernelGGL((k_hb_embed<T>), dim3(n), dim3(256), 0, st, (const T*)m->w.embedding, ids, 1, m->xa, m->xb, W, c.vocab, c.embed_scale, bg,
+                       io->pos, io->row_req, io->req_rows, io->req_state);
+    if (bigram && n != n_req)
+        hipLaunchKernelGGL(k_hb_store_prev, dim3((n_req + 63) / 64), dim3(64), 0, st, ids, 1, c.vocab, io->req_rows, io->req_state, m->w.prev_token, n_req);
     float *cur = m->xa, *other = m->xb;
     for (int ri = 0; ri < c.n_runs; ++ri) {
         const vox_hybrid_run& run = m->runs[ri];
@@ -2206,22 +2540,31 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             float* t = cur; cur = other; other = t;
         }
         const bool has_ff = L.ff > 0 || L.moe;
-        const bool parallel = L.block == VOX_BLOCK_PARALLEL;
+        const bool one_norm = L.block == VOX_BLOCK_PARALLEL_ONE_NORM;
+        const bool parallel = L.block == VOX_BLOCK_PARALLEL || one_norm;
         // a parallel layer norms x once for both branches before anything is added; a mixer with a sibling needs the normed rows twice
         const float* hn = nullptr;
         if (parallel || L.sibling >= 0) {
-            hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, parallel && has_ff ? L.norm2 : nullptr, m->h2, (long)W);
+            hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, parallel && has_ff && !one_norm ? L.norm2 : nullptr, m->h2, (long)W);
             hn = m->h;
         }
+        const float* hf = one_norm ? m->h : m->h2;      // what the feed-forward of a parallel layer reads
         VOX_TRY(hb_mixer<T>(m, st, io, L, run.cache, run.pool, run.state, hn, cur, ldx, n, n_req, max_kvlen));
         if (L.sibling >= 0)
             VOX_TRY(hb_mixer<T>(m, st, io, m->layers[L.sibling], run.side_cache, run.side_pool, run.side_state, hn, cur, ldx, n, n_req, max_kvlen));
         if (L.moe) {
             if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
-            VOX_TRY(hb_moe<T>(m, st, *L.moe, m->h2, cur, ldx, n));
+            VOX_TRY(hb_moe<T>(m, st, *L.moe, hf, cur, ldx, n));
+        } else if (L.ff > 0 && L.ff_kind == VOX_FF_GATED) {
+            // down(act(gate h + b) * (up h + b)) + b: gate and up rows in one product, the activation in place behind it
+            if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, hf, W, (const T*)L.w_up, L.b_up, m->ff, 2 * L.ff, n, 2 * L.ff, W));
+            hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (L.ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->ff_act, L.ff, INFINITY, 1.0f,
+                               (const int*)nullptr, 0, 0.0f, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0);
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff_act, L.ff, (const T*)L.w_down, L.b_down, cur, ldx, n, W, L.ff));
         } else if (L.ff > 0) {
             if (parallel) {
-                VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h2, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
+                VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, hf, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
             } else if (!(n == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_GELU, cur, ldx, nullptr, L.norm2, (const T*)L.w_up, nullptr, m->ff, L.ff, W))) {
                 hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h, nullptr, nullptr, (long)W);
                 VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
@@ -2232,10 +2575,13 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        if (!(n_out == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr,
-                                                io->logits, c.vocab, W))) {
+        if (!(n_out == 1 && !(c.logit_softcap > 0.f) &&
+              hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr, io->logits, c.vocab, W))) {
             hb_norm(m, st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, nullptr, nullptr, (long)W);
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
+            hb_rowmap rm = hb_plain();
+            rm.epi_arg = c.logit_softcap;
+            VOX_TRY(hb_gemm<T>(st, c.logit_softcap > 0.f ? HB_EPI_SOFTCAP : HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits,
+                               c.vocab, n_out, c.vocab, W, rm));
         }
     }
     VOX_HIP(hipGetLastError());
@@ -2267,17 +2613,26 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         else if (L.heads < 1 || L.dim < 1 || L.vdim < 1) bad = "heads / dim / vdim";
         else if (L.vdim > 64 * HB_MAX_VPL && L.kind != VOX_MIXER_RGLRU) bad = "vdim above 512";
         else if (!L.norm1 || !L.w_in || !L.w_out) bad = "missing weights";
-        else if (L.ff > 0 && (!L.norm2 || !L.w_up || !L.w_down)) bad = "missing feed-forward weights";
-        else if (L.block != VOX_BLOCK_SEQUENTIAL && L.block != VOX_BLOCK_PARALLEL) bad = "block form";
+        else if (L.ff > 0 && ((!L.norm2 && L.block != VOX_BLOCK_PARALLEL_ONE_NORM) || !L.w_up || !L.w_down)) bad = "missing feed-forward weights";
+        else if (L.ff > 0 && L.ff_kind != VOX_FF_UP_DOWN && L.ff_kind != VOX_FF_GATED) bad = "feed-forward form";
+        else if (L.block != VOX_BLOCK_SEQUENTIAL && L.block != VOX_BLOCK_PARALLEL && L.block != VOX_BLOCK_PARALLEL_ONE_NORM) bad = "block form";
         else if (L.sibling >= cfg->n_layers || (L.sibling >= 0 && m->layers[L.sibling].sibling >= 0)) bad = "sibling index";
         else if (L.kind == VOX_MIXER_HGRN2 && (!L.lower || !L.head_norm)) bad = "hgrn2 needs lower and head_norm";
         else if (L.kind == VOX_MIXER_MLSTM && (!L.head_norm || !(L.gate_cap > 0.f))) bad = "mlstm needs head_norm and gate_cap";
-        else if ((L.kind == VOX_MIXER_HGRN2 || L.kind == VOX_MIXER_MLSTM || L.kind == VOX_MIXER_SHIFT_DECAY) && L.dim > 64 * HB_SCAN_MAX_WAVES)
+        else if (L.kind == VOX_MIXER_RETENTION && (!L.decay || L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)))
+            bad = "retention needs decay and an even rot_dims <= dim";
+        else if (L.kind == VOX_MIXER_LATENT_ATTN) {
+            if (L.q_rank < 1 || L.kv_rank < 1 || L.rot_dim < 0 || !L.w_uq || !L.w_ukT || !L.w_uv || !L.q_lat_norm || !L.kv_lat_norm) bad = "latent attention: ranks / expansions / norms";
+            else if (L.kv_rank > 64 * HB_MAX_VPL) bad = "latent attention: kv_rank above 512";
+            else if (L.rot_dims < 0 || L.rot_dims > L.rot_dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)) bad = "latent attention: rot_dims";
+            else if (L.window < 0) bad = "latent attention: window";
+        }
+        else if ((L.kind == VOX_MIXER_HGRN2 || L.kind == VOX_MIXER_MLSTM || L.kind == VOX_MIXER_SHIFT_DECAY || L.kind == VOX_MIXER_RETENTION) && L.dim > 64 * HB_SCAN_MAX_WAVES)
             bad = "recurrent dim above 1024";
         else if (L.kind == VOX_MIXER_RGLRU && (L.dim != L.vdim || L.conv_taps < 1 || !L.conv_w || !L.w_gates || !L.lam)) bad = "rglru needs conv, gates and lam";
         else if (L.kind == VOX_MIXER_SHIFT_DECAY && (L.dim != L.vdim || L.lora < 1 || !L.shift_mu || !L.w_decay2 || !L.decay0 || !L.bonus || !L.head_norm))
             bad = "shift-decay needs mu, decay and bonus tensors";
-        else if (hb_is_attn(L.kind)) {
+        else if (hb_is_attn(L.kind) && L.kind != VOX_MIXER_LATENT_ATTN) {
             if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || L.heads / L.kv_heads > 16) bad = "heads / kv_heads (group of at most 16)";
             else if (L.dim > 64 * HB_MAX_DPL) bad = "dim above 512";
             else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && (L.window < 1 || L.pool < 1)) bad = "window / pool";
@@ -2286,7 +2641,8 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         if (!bad && L.moe) {
             const vox_hybrid_moe& E = *L.moe;
             if (E.experts < 0 || E.identity < 0 || E.top < 1 || E.top > E.experts + E.identity) bad = "moe: experts / identity / top";
-            else if (!E.router || !L.norm2) bad = "moe: router or norm2 missing";
+            else if (!E.router || (!L.norm2 && L.block != VOX_BLOCK_PARALLEL_ONE_NORM)) bad = "moe: router or norm2 missing";
+            else if (E.score_kind != VOX_ROUTER_SOFTMAX && E.score_kind != VOX_ROUTER_SIGMOID) bad = "moe: score kind";
             else if (E.experts > 0 && (E.ff < 1 || !E.w_gate_up || !E.w_down)) bad = "moe: expert weights";
             else if (E.shared_ff > 0 && (!E.shared_gate_up || !E.shared_down)) bad = "moe: shared expert weights";
         }
@@ -2294,7 +2650,12 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         const int n_proj = hb_layer_proj(L);
         if (n_proj > m->max_in) m->max_in = n_proj;
         if (L.heads * L.vdim > m->max_mix) m->max_mix = L.heads * L.vdim;
-        if (L.ff > m->max_ff) m->max_ff = L.ff;
+        if ((L.ff_kind == VOX_FF_GATED ? 2 : 1) * L.ff > m->max_ff) m->max_ff = (L.ff_kind == VOX_FF_GATED ? 2 : 1) * L.ff;
+        if (L.ff_kind == VOX_FF_GATED && L.ff > m->max_gated) m->max_gated = L.ff;
+        if (L.kind == VOX_MIXER_RETENTION) {
+            const size_t f = ((size_t)cfg->max_rows / HB_SCAN_CHUNK + cfg->max_batch + 1) * L.heads * ((size_t)L.dim * L.vdim);
+            if (f > m->scan_ws_floats) m->scan_ws_floats = f;
+        }
         if (L.kind == VOX_MIXER_SHIFT_DECAY) {
             m->any_shift = true;
             const size_t f = ((size_t)cfg->max_rows / HB_SCAN_CHUNK + cfg->max_batch + 1) * L.heads * ((size_t)L.dim * L.dim + L.dim);
@@ -2317,6 +2678,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         else {
             const vox_hybrid_layer& L = m->layers[r.layer];
             if (hb_is_attn(L.kind) ? (!r.cache || (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.pool)) : !r.state) bad = "missing cache / state";
+            else if (cfg->bigram_buckets > 0 && (!w->bigram || !w->prev_token)) bad = "bigram table / previous-token state";
             else if (L.sibling >= 0) {
                 const vox_hybrid_layer& S2 = m->layers[L.sibling];
                 if (hb_is_attn(S2.kind) ? (!r.side_cache || (S2.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.side_pool)) : !r.side_state)
@@ -2335,6 +2697,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
               hipMalloc((void**)&m->hout, (size_t)cfg->max_out * W * 4) == hipSuccess &&
               hipMalloc((void**)&m->logits16, (size_t)cfg->max_batch * cfg->vocab * 2) == hipSuccess;
     if (ok && m->any_shift) ok = hipMalloc((void**)&m->shift, 5 * R * W * 4) == hipSuccess;
+    if (ok && m->max_gated) ok = hipMalloc((void**)&m->ff_act, R * (size_t)m->max_gated * 4) == hipSuccess;
     if (ok && m->scan_ws_floats && cfg->max_rows > HB_SCAN_CHUNK) ok = hipMalloc((void**)&m->scan_ws, m->scan_ws_floats * 4) == hipSuccess;
     if (ok && m->max_top > 0) {
         const size_t ne = R * (size_t)m->max_top;
@@ -2349,10 +2712,11 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
     // partial results of segmented attention launches: few rows x heads x segments of the longest sequence
     for (const vox_hybrid_layer& L : m->layers)
         if (hb_is_attn(L.kind)) {
-            const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN;
-            const int max_keys = causal ? cfg->max_seq_len : (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + cfg->max_seq_len / L.pool + 1;
+            const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN, latent = L.kind == VOX_MIXER_LATENT_ATTN;
+            const int max_keys = causal || (latent && L.window < 1) ? cfg->max_seq_len
+                                 : (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + (latent ? 0 : cfg->max_seq_len / L.pool + 1);
             const size_t nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
-            const size_t b = (size_t)HB_ATTN_SEG_ROWS * L.heads * nseg * (L.vdim + 2) * 4;
+            const size_t b = (size_t)HB_ATTN_SEG_ROWS * L.heads * nseg * ((latent ? L.kv_rank : L.vdim) + 2) * 4;
             if (b > m->attn_ws_bytes) m->attn_ws_bytes = b;
         }
     if (ok && m->attn_ws_bytes) ok = hipMalloc((void**)&m->attn_ws, m->attn_ws_bytes) == hipSuccess;
@@ -2364,7 +2728,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
 void vox_hybrid_destroy(vox_hybrid* m) {
     if (!m) return;
     (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->h2); (void)hipFree(m->proj); (void)hipFree(m->mix);
-    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift); (void)hipFree(m->scan_ws);
+    (void)hipFree(m->ff); (void)hipFree(m->ff_act); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift); (void)hipFree(m->scan_ws);
     (void)hipFree(m->moe_wgt); (void)hipFree(m->moe_sel); (void)hipFree(m->moe_act); (void)hipFree(m->moe_out);
     (void)hipFree(m->moe_list); (void)hipFree(m->moe_count);
     delete m;

@@ -1,6 +1,7 @@
 """Host side of `vox_hybrid_*`: the engine for decoders that mix tokens with linear recurrences (HGRN2, mLSTM, a real-gated
-diagonal unit behind a short convolution, a matrix state with token shift and per-channel decay) and with attention over a paged
-cache (a sliding window with pooled history, or plain causal attention with normed q / k / v), optionally two mixers side by
+diagonal unit behind a short convolution, a matrix state with token shift and per-channel decay, retention with a fixed decay
+per head) and with attention over a paged cache (a sliding window with pooled history, plain causal attention with normed
+q / k / v, or windowed attention whose keys and values are expanded from a cached low-rank latent), optionally two mixers side by
 side, sequential or parallel layers, a dense or a routed feed-forward, and a range of layers looped over shared weights.
 
 It reuses the plan / stream / hipGraph machinery of the other LM engines (`Qwen3Engine`): one pinned int32 plan block per
@@ -20,11 +21,16 @@ from . import _native as N
 from .engine import Qwen3Engine
 
 MIXER_HGRN2, MIXER_POOLED_WINDOW_ATTN, MIXER_MLSTM, MIXER_RGLRU, MIXER_CAUSAL_ATTN, MIXER_SHIFT_DECAY = 0, 1, 2, 3, 4, 5
+MIXER_LATENT_ATTN, MIXER_RETENTION = 6, 7
 MIXER_KINDS = {"hgrn2": MIXER_HGRN2, "attention": MIXER_POOLED_WINDOW_ATTN, "mlstm": MIXER_MLSTM, "rglru": MIXER_RGLRU,
-               "causal_attention": MIXER_CAUSAL_ATTN, "shift_decay": MIXER_SHIFT_DECAY}
-ATTENTION_KINDS = ("attention", "causal_attention")
+               "causal_attention": MIXER_CAUSAL_ATTN, "shift_decay": MIXER_SHIFT_DECAY, "latent_attention": MIXER_LATENT_ATTN,
+               "retention": MIXER_RETENTION}
+ATTENTION_KINDS = ("attention", "causal_attention", "latent_attention")
 NORM_KINDS = {"layer": 0, "rms_groups": 1}
-BLOCK_FORMS = {"sequential": 0, "parallel": 1}
+BLOCK_FORMS = {"sequential": 0, "parallel": 1, "parallel_one_norm": 2}
+FF_KINDS = {"up_down": 0, "gated": 1}
+ACT_KINDS = {"gelu_tanh": 0, "swish": 1}
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
 
 
 @dataclass
@@ -38,6 +44,10 @@ class MoECfg:
     shared_ff: int = 0
     shared_limit: float = 0.0
     act_alpha: float = 1.702
+    score: str = "softmax"          # "softmax" over all router outputs | "sigmoid" of each
+    renorm: bool = True             # weights divided by the sum of the chosen scores
+    scale_input: bool = False       # the weight multiplies what the expert reads, not what it returns
+    up_offset: float = 1.0          # y = g * sigmoid(act_alpha g) * (u + up_offset)
 
 
 @dataclass
@@ -63,6 +73,13 @@ class MixerCfg:
     lora: int = 0                   # shift_decay: width of the decay bottleneck
     out_scale: float = 1.0          # the mixer's output is multiplied by this before it joins the residual sum
     block: str = "sequential"       # "sequential": x += mixer(norm1 x); x += ff(norm2 x) | "parallel": x += mixer(norm1 x) + ff(norm2 x)
+                                    # | "parallel_one_norm": x += mixer(n) + ff(n), n = norm1 x
+    ff_kind: str = "up_down"        # dense feed-forward: "up_down" down(gelu(up h)) | "gated" down(act(gate h + b) * (up h + b)) + b
+    ff_act: str = "gelu_tanh"       # activation of the gated form ("gelu_tanh" | "swish")
+    q_rank: int = 0                 # latent attention: width of the query latent
+    kv_rank: int = 0                # latent attention: width of the cached key / value latent
+    rot_dim: int = 0                # latent attention: rotated query / key dims per head (the key part is shared by all heads)
+    decay: Optional[List[float]] = None     # retention: one decay per head
     side: Optional["MixerCfg"] = None   # a second mixer on the same normed input, added to the same sum
     moe: Optional[MoECfg] = None    # routed feed-forward (instead of the dense one)
 
@@ -80,13 +97,23 @@ class MixerCfg:
             return h * d + self.kv_heads * (d + v)
         if self.kind == "shift_decay":
             return 4 * h * d + self.lora
+        if self.kind == "latent_attention":
+            return self.q_rank + self.kv_rank + self.rot_dim + h
+        if self.kind == "retention":
+            return 2 * h * d + 2 * h * v
         return 2 * h * d + 2 * h * v + 2 * h
+
+    def cache_values(self) -> int:
+        """Values one token leaves in the paged cache of an attention mixer."""
+        if self.kind == "latent_attention":
+            return self.kv_rank + self.rot_dim
+        return self.kv_heads * (self.dim + self.vdim) if self.kind in ATTENTION_KINDS else 0
 
     def state_floats(self, width: int) -> int:
         """fp32 values of one recurrent-state slot (0 for attention)."""
         h, d, v = self.heads, self.dim, self.vdim
         return {"hgrn2": h * d * v, "mlstm": h * (d * v + d + 1), "rglru": max(self.conv_taps, 1) * h * d,
-                "shift_decay": h * d * d + width}.get(self.kind, 0)
+                "shift_decay": h * d * d + width, "retention": h * d * v}.get(self.kind, 0)
 
 
 @dataclass
@@ -99,6 +126,8 @@ class HybridCfg:
     norm_kind: str = "layer"        # "layer": weight-only layer norm | "rms_groups": RMS norm over norm_groups equal slices
     norm_groups: int = 1
     embed_scale: float = 1.0
+    logit_softcap: float = 0.0      # > 0: logits <- cap * tanh(logits / cap)
+    bigram: Optional[tuple] = None  # (buckets, mul_prev, mul_cur): x0 += bigram[(prev * mul_prev + id * mul_cur) mod buckets]
 
     def runs(self):
         """[(layer index, loop_in)] in execution order; loop_in marks the first layer of every pass of the looped range."""
@@ -115,7 +144,8 @@ class HybridCfg:
 class HybridMoEC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("experts", "identity", "top", "ff", "shared_ff")] + \
                [(n, ctypes.c_float) for n in ("limit", "shared_limit", "act_alpha")] + \
-               [(n, ctypes.c_void_p) for n in ("router", "correction", "w_gate_up", "w_down", "shared_gate_up", "shared_down")]
+               [(n, ctypes.c_void_p) for n in ("router", "correction", "w_gate_up", "w_down", "shared_gate_up", "shared_down")] + \
+               [(n, ctypes.c_int32) for n in ("score_kind", "renorm", "scale_input")] + [("up_offset", ctypes.c_float)]
 
 
 class HybridLayerC(ctypes.Structure):
@@ -129,7 +159,11 @@ class HybridLayerC(ctypes.Structure):
                 ("conv_taps", ctypes.c_int32), ("rec_scale", ctypes.c_float), ("conv_w", ctypes.c_void_p), ("conv_b", ctypes.c_void_p),
                 ("w_gates", ctypes.c_void_p), ("b_gates", ctypes.c_void_p), ("lam", ctypes.c_void_p),
                 ("lora", ctypes.c_int32), ("shift_mu", ctypes.c_void_p), ("w_decay2", ctypes.c_void_p), ("decay0", ctypes.c_void_p),
-                ("bonus", ctypes.c_void_p), ("moe", ctypes.POINTER(HybridMoEC))]
+                ("bonus", ctypes.c_void_p), ("moe", ctypes.POINTER(HybridMoEC)),
+                ("ff_kind", ctypes.c_int32), ("ff_act", ctypes.c_int32), ("b_up", ctypes.c_void_p), ("b_down", ctypes.c_void_p),
+                ("q_rank", ctypes.c_int32), ("kv_rank", ctypes.c_int32), ("rot_dim", ctypes.c_int32),
+                ("w_uq", ctypes.c_void_p), ("w_ukT", ctypes.c_void_p), ("w_uv", ctypes.c_void_p),
+                ("q_lat_norm", ctypes.c_void_p), ("kv_lat_norm", ctypes.c_void_p), ("decay", ctypes.c_void_p)]
 
 
 class HybridRunC(ctypes.Structure):
@@ -141,12 +175,14 @@ class HybridRunC(ctypes.Structure):
 class HybridConfigC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("width", "vocab", "n_layers", "n_runs", "dtype", "page_size", "max_rows",
                                               "max_batch", "max_out", "max_pages", "max_seq_len")] + [("eps", ctypes.c_float)] + \
-               [("norm_kind", ctypes.c_int32), ("norm_groups", ctypes.c_int32), ("embed_scale", ctypes.c_float)]
+               [("norm_kind", ctypes.c_int32), ("norm_groups", ctypes.c_int32), ("embed_scale", ctypes.c_float),
+                ("logit_softcap", ctypes.c_float), ("bigram_buckets", ctypes.c_int32), ("bigram_mul_prev", ctypes.c_int32),
+                ("bigram_mul_cur", ctypes.c_int32)]
 
 
 class HybridWeightsC(ctypes.Structure):
     _fields_ = [("layers", ctypes.POINTER(HybridLayerC)), ("runs", ctypes.POINTER(HybridRunC))] + \
-               [(n, ctypes.c_void_p) for n in ("embedding", "loop_in", "head", "final_norm")]
+               [(n, ctypes.c_void_p) for n in ("embedding", "loop_in", "head", "final_norm", "bigram", "prev_token")]
 
 
 class HybridIO(ctypes.Structure):
@@ -161,12 +197,15 @@ def rotary_frequencies(rot_dims: int, base: float, factor: float) -> torch.Tenso
     return torch.pow(torch.tensor(base, dtype=torch.float32), -(2.0 * i) / rot_dims) / factor
 
 
+ROTARY_KINDS = ("attention", "latent_attention", "retention")
+
+
 class HybridEngine(Qwen3Engine):
     """`weights`: {"embedding", "head", "final_norm", "loop_in" (or None), "layers": [per layer dict with norm1, norm2, w_in,
-    b_in, w_out, lower, head_norm, w_up, w_down; per mixer kind also q_norm, k_norm | conv_w, conv_b, w_gates, b_gates, lam |
-    shift_mu, w_decay2, decay0, bonus; "moe": {router, correction, w_gate_up, w_down, shared_gate_up, shared_down}; "side":
-    the same mixer keys for a sibling mixer]} — matrices in any float dtype (stored as the engine's dtype), vectors and
-    the router stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
+    b_in, w_out, lower, head_norm, w_up, w_down, b_up, b_down; per mixer kind also q_norm, k_norm | conv_w, conv_b, w_gates, b_gates,
+    lam | shift_mu, w_decay2, decay0, bonus | w_uq, w_ukT, w_uv, q_lat_norm, kv_lat_norm; "moe": {router, correction, w_gate_up,
+    w_down, shared_gate_up, shared_down}; "side": the same mixer keys for a sibling mixer], "bigram" (or None)} — matrices in any
+    float dtype (stored as the engine's dtype), vectors and the router stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
 
     needs_state_slots = True
 
@@ -212,7 +251,7 @@ class HybridEngine(Qwen3Engine):
             c.norm1, c.norm2 = vec(lw["norm1"]), vec(lw.get("norm2"))
             c.w_in, c.b_in, c.w_out = mat(lw["w_in"]), vec(lw.get("b_in")), mat(lw["w_out"])
             c.lower, c.head_norm = vec(lw.get("lower")), vec(lw.get("head_norm"))
-            c.inv_freq = vec(rotary_frequencies(m.rot_dims, m.rot_base, m.rot_factor)) if m.kind == "attention" and m.rot_dims else None
+            c.inv_freq = vec(rotary_frequencies(m.rot_dims, m.rot_base, m.rot_factor)) if m.kind in ROTARY_KINDS and m.rot_dims else None
             c.w_up, c.w_down = mat(lw.get("w_up")), mat(lw.get("w_down"))
             c.block, c.sibling, c.out_scale = BLOCK_FORMS[m.block], -1, m.out_scale
             c.q_norm, c.k_norm = vec(lw.get("q_norm")), vec(lw.get("k_norm"))
@@ -222,11 +261,20 @@ class HybridEngine(Qwen3Engine):
                 vec(lw.get("b_gates")), vec(lw.get("lam"))
             c.lora, c.shift_mu, c.w_decay2 = m.lora, vec(lw.get("shift_mu")), mat(lw.get("w_decay2"))
             c.decay0, c.bonus = vec(lw.get("decay0")), vec(lw.get("bonus"))
+            c.ff_kind, c.ff_act, c.b_up, c.b_down = FF_KINDS[m.ff_kind], ACT_KINDS[m.ff_act], vec(lw.get("b_up")), vec(lw.get("b_down"))
+            c.q_rank, c.kv_rank, c.rot_dim = m.q_rank, m.kv_rank, m.rot_dim
+            c.w_uq, c.w_ukT, c.w_uv = mat(lw.get("w_uq")), mat(lw.get("w_ukT")), mat(lw.get("w_uv"))
+            c.q_lat_norm, c.kv_lat_norm = vec(lw.get("q_lat_norm")), vec(lw.get("kv_lat_norm"))
+            if m.kind == "retention":
+                if m.decay is None or len(m.decay) != m.heads:
+                    raise ValueError(f"layer {i}: retention needs one decay per head")
+                c.decay = vec(torch.tensor([float(a) for a in m.decay], dtype=torch.float32))
             if m.moe is not None:
                 e, ew = m.moe, lw["moe"]
                 mc = HybridMoEC(e.experts, e.identity, e.top, e.ff, e.shared_ff, e.limit, e.shared_limit, e.act_alpha,
                                 vec(ew["router"]), vec(ew.get("correction")), mat(ew.get("w_gate_up")), mat(ew.get("w_down")),
-                                mat(ew.get("shared_gate_up")), mat(ew.get("shared_down")))
+                                mat(ew.get("shared_gate_up")), mat(ew.get("shared_down")), ROUTER_SCORES[e.score], int(e.renorm),
+                                int(e.scale_input), e.up_offset)
                 self._moes.append(mc)
                 c.moe = ctypes.pointer(mc)
 
@@ -243,7 +291,7 @@ class HybridEngine(Qwen3Engine):
         def storage(m):
             """(cache, pool, state) of one mixer of one run."""
             if m.kind in ATTENTION_KINDS:
-                kv = torch.zeros(max_pages * page_size * m.kv_heads * (m.dim + m.vdim), dtype=dtype, device=dev)
+                kv = torch.zeros(max_pages * page_size * m.cache_values(), dtype=dtype, device=dev)
                 self.caches.append(kv)
                 if m.kind == "attention":
                     pool = torch.zeros(max_pages, (page_size - 1) // m.pool + 1, m.kv_heads, m.dim + m.vdim, dtype=torch.float32, device=dev)
@@ -261,11 +309,19 @@ class HybridEngine(Qwen3Engine):
             if m.side is not None:
                 rarr[j].side_cache, rarr[j].side_pool, rarr[j].side_state = storage(m.side)
         self.n_runs = len(runs)
+        bg = cfg.bigram or (0, 0, 0)
         cc = HybridConfigC(W, cfg.vocab, len(larr), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
                            max_batch, self.max_out, max_pages, max_seq_len, cfg.eps, NORM_KINDS[cfg.norm_kind], cfg.norm_groups,
-                           cfg.embed_scale)
+                           cfg.embed_scale, cfg.logit_softcap, int(bg[0]), int(bg[1]), int(bg[2]))
+        # the last token every state slot's sequence has seen (what a bigram embedding needs of the step before)
+        self.prev_token = torch.zeros(self.state_slots, dtype=torch.int32, device=dev)
+        if cfg.bigram and tuple(weights["bigram"].shape) != (int(bg[0]) + 1, W):
+            raise ValueError(f"bigram table {tuple(weights['bigram'].shape)}: expected {(int(bg[0]) + 1, W)}")
+        emb = mat(weights["embedding"])
+        head = emb if weights["head"] is weights["embedding"] else mat(weights["head"])      # a tied head shares the table
         cw = HybridWeightsC(ctypes.cast(larr, ctypes.POINTER(HybridLayerC)), ctypes.cast(rarr, ctypes.POINTER(HybridRunC)),
-                            mat(weights["embedding"]), mat(weights.get("loop_in")), mat(weights["head"]), vec(weights["final_norm"]))
+                            emb, mat(weights.get("loop_in")), head, vec(weights["final_norm"]),
+                            mat(weights.get("bigram")) if cfg.bigram else None, self.prev_token.data_ptr())
         self._larr, self._rarr = larr, rarr
         h = ctypes.c_void_p()
         N.check(L.vox_hybrid_create(self.ctx, ctypes.byref(cc), ctypes.byref(cw), ctypes.byref(h)))
@@ -307,7 +363,7 @@ class HybridEngine(Qwen3Engine):
 
     def _mutable_state(self):
         # a decode step advances the recurrent states and appends K / V: the warm-up run before a capture must leave no trace
-        return [self.input_ids, self.rng_offset] + self.states
+        return [self.input_ids, self.rng_offset, self.prev_token] + self.states
 
     def _native_frame(self, io, st, batch, bucket, sampling, seed, feedback):
         N.check(self.L.vox_hybrid_step(self.h, st, ctypes.byref(io), self.input_ids.data_ptr(), batch, batch, batch, int(bucket),

@@ -191,6 +191,12 @@ def _fusanex(model_name, device="cuda:0", weights=None, checkpoint_dir=None, syn
     return _hybrid_lm(".fusanex", "FusanexModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
 
 
+@register_model("dipivik")
+def _dipivik(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
+    """One-norm parallel-block LM of latent attention and retention layers with gated dense or sigmoid-routed feed-forwards."""
+    return _hybrid_lm(".dipivik", "DipivikModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
+
+
 def load_checkpoint_dir(path: str, device: str = "cuda:0", **kw):
     """A local checkpoint folder whose config.json names its architecture: the registry entry of that name loads it."""
     import json
