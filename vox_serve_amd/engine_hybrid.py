@@ -200,6 +200,17 @@ def rotary_frequencies(rot_dims: int, base: float, factor: float) -> torch.Tenso
 ROTARY_KINDS = ("attention", "latent_attention", "retention")
 
 
+def reduced_bigram(bigram) -> tuple:
+    """(buckets, mul_prev, mul_cur) with the multipliers taken modulo the bucket count (the hash is unchanged, every product of a
+    token id and a multiplier stays far inside 64 bits); (0, 0, 0) for none."""
+    if not bigram:
+        return (0, 0, 0)
+    n, a, b = (int(v) for v in bigram)
+    if n < 1 or n >= 1 << 31:
+        raise ValueError(f"bigram buckets {n}")
+    return (n, a % n, b % n)
+
+
 class HybridEngine(Qwen3Engine):
     """`weights`: {"embedding", "head", "final_norm", "loop_in" (or None), "layers": [per layer dict with norm1, norm2, w_in,
     b_in, w_out, lower, head_norm, w_up, w_down, b_up, b_down; per mixer kind also q_norm, k_norm | conv_w, conv_b, w_gates, b_gates,
@@ -309,7 +320,7 @@ class HybridEngine(Qwen3Engine):
             if m.side is not None:
                 rarr[j].side_cache, rarr[j].side_pool, rarr[j].side_state = storage(m.side)
         self.n_runs = len(runs)
-        bg = cfg.bigram or (0, 0, 0)
+        bg = reduced_bigram(cfg.bigram)
         cc = HybridConfigC(W, cfg.vocab, len(larr), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
                            max_batch, self.max_out, max_pages, max_seq_len, cfg.eps, NORM_KINDS[cfg.norm_kind], cfg.norm_groups,
                            cfg.embed_scale, cfg.logit_softcap, int(bg[0]), int(bg[1]), int(bg[2]))
