@@ -743,11 +743,18 @@ def main():
     ap.add_argument("--sirodra", action="store_true", help="instead of the default workload: prefill / decode throughput of the hybrid-mixer "
                     "engine (Sirodra layer pattern, random weights) beside the single-stack LM engine at equal width and depth "
                     "(tools/bench_sirodra.py); prints that comparison as one JSON line")
+    ap.add_argument("--dipivik", action="store_true", help="instead of the default workload: prefill / decode throughput of the Dipivik "
+                    "design (random weights) beside Fusanex, the closest existing model, on the same engine at equal width and depth "
+                    "(tools/bench_dipivik.py); prints that comparison as one JSON line")
     ap.add_argument("--fusanex", action="store_true", help="instead of the default workload: prefill / decode throughput of the Fusanex "
                     "design (random weights) beside Sirodra, the closest existing model, on the same engine at equal width and depth "
                     "(tools/bench_fusanex.py); prints that comparison as one JSON line")
     args = ap.parse_args()
 
+    if args.dipivik:
+        from tools.bench_dipivik import run as run_dipivik
+        print(json.dumps(run_dipivik(steps=min(args.steps, 50), warmup=min(args.warmup, 10))))
+        return
     if args.fusanex:
         from tools.bench_fusanex import run as run_fusanex
         print(json.dumps(run_fusanex(steps=min(args.steps, 50), warmup=min(args.warmup, 10))))

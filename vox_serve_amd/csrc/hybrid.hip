@@ -1886,12 +1886,12 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
 
 // few-row steps: the segments' partial results of a (row, head), merged in segment order; output gate applied here
 __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, float* out, long ldo, const int* pos, int H, int vdim,
-                                                      int window, int P, int seg_chunks, const float* gate, long ldg, float out_scale) {
+                                                      int window, int P, int seg_chunks, const float* gate, long ldg, float out_scale, int chunk) {
     const int row = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
     const int p = pos[row];
     const int first = p - window + 1;
     const int total = (first > 0 ? first / P : 0) + (p - (first > 0 ? first : 0) + 1);
-    const int nseg = (((total + 63) >> 6) + seg_chunks - 1) / seg_chunks;
+    const int nseg = ((total + chunk - 1) / chunk + seg_chunks - 1) / seg_chunks;
     const float* src = part + (size_t)(row * H + hq) * nseg_grid * (vdim + 2);
     float mm = -INFINITY;
     for (int s2 = 0; s2 < nseg; ++s2) mm = fmaxf(mm, src[(size_t)s2 * (vdim + 2) + vdim]);
@@ -1903,6 +1903,182 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
         for (int s2 = 0; s2 < nseg; ++s2) a += src[(size_t)s2 * (vdim + 2) + j] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
         out[(size_t)row * ldo + hq * vdim + j] = a / lt * gmul;
     }
+}
+
+// ---- latent attention, steps of few rows: one block per (row, segment of keys), every head against a key tile held in LDS ------
+// All heads read the same cached rows [R latent | r rotated key part]; the first R values are also the value.  The block stages KT
+// keys at a time in LDS (as the cache holds them), every thread takes one key and HPT heads for the scores (fp32 sums over the dims in
+// ascending order), the weights of a (head, tile) come from one running softmax per head, then every thread owns two value columns of
+// all heads of the group.  Heads are taken in groups of 16.  part != NULL: the block leaves an unnormalised partial result per head
+// (k_hb_attn_merge's layout) for its `cpb` tiles; else it covers all keys and writes o / l * sigmoid(gate) * out_scale.
+#define HB_LAT_HG 16
+template <typename T> struct hb_lat_tile { static constexpr int KT = sizeof(T) == 2 ? 64 : 32; };
+template <typename T>
+__global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, long ldq, const T* cache, float* out, long ldo, const int* pos,
+                                                             const int* row_req, const int* ptab, int pts, int H, int R, int r, int window,
+                                                             int ps, float scale, int cpb, float* part, const float* gate, long ldg,
+                                                             float out_scale, int DP) {
+    constexpr int KT = hb_lat_tile<T>::KT, NS = 256 / KT, HPT = HB_LAT_HG / NS;
+    extern __shared__ float sm[];
+    const int D = R + r, Dq = (D + 3) & ~3;
+    T* Kt = (T*)sm;                                                    // [KT][DP]
+    float* qs = sm + (((size_t)KT * DP * sizeof(T) + 15) / 16) * 4;    // [16][Dq]
+    float* pw = qs + HB_LAT_HG * Dq;                                   // [KT][16] weights of the tile
+    float* al = pw + KT * HB_LAT_HG;                                   // [16] rescale factors of the tile
+    float* ml = al + HB_LAT_HG;                                        // [16][2] final maximum and sum
+    const int row = blockIdx.x, seg = blockIdx.y, tid = threadIdx.x;
+    const int p = pos[row];
+    const int* pt = ptab + (size_t)row_req[row] * pts;
+    const int lo = p - window + 1 > 0 ? p - window + 1 : 0;
+    const int total = p - lo + 1, nchunks = (total + KT - 1) / KT;
+    const int c0 = seg * cpb, c1 = c0 + cpb < nchunks ? c0 + cpb : nchunks;
+    if (c0 >= nchunks) return;
+    const int j = tid % KT, hs = tid / KT;
+    constexpr int VE = 16 / sizeof(T);
+    const bool vec = (D % VE == 0) && ((((size_t)cache) & 15) == 0);
+    const bool quad = (D % 4 == 0);
+    for (int h0 = 0; h0 < H; h0 += HB_LAT_HG) {
+        const int hg = H - h0 < HB_LAT_HG ? H - h0 : HB_LAT_HG;
+        __syncthreads();
+        for (int i = tid; i < HB_LAT_HG * Dq; i += 256) {
+            const int h = i / Dq, d = i - h * Dq;
+            qs[i] = (h < hg && d < D) ? qa[(size_t)row * ldq + (size_t)(h0 + h) * D + d] : 0.f;
+        }
+        float m[HPT], l[HPT], acc[HB_LAT_HG][2];
+#pragma unroll
+        for (int i = 0; i < HPT; ++i) { m[i] = -INFINITY; l[i] = 0.f; }
+#pragma unroll
+        for (int h = 0; h < HB_LAT_HG; ++h) acc[h][0] = acc[h][1] = 0.f;
+        for (int c = c0; c < c1; ++c) {
+            const int base = c * KT, cnt = total - base < KT ? total - base : KT;
+            __syncthreads();
+            // the tile: key jj of the tile is the token at position lo + base + jj; rows behind the last key are zero
+            if (vec) {
+                const int per = D / VE;
+                for (int idx = tid; idx < KT * per; idx += 256) {
+                    const int jj = idx / per, v = idx - jj * per;
+                    uint4 u = make_uint4(0, 0, 0, 0);
+                    if (jj < cnt) {
+                        const int t = lo + base + jj;
+                        u = *(const uint4*)(cache + ((size_t)pt[t / ps] * ps + t % ps) * (size_t)D + (size_t)v * VE);
+                    }
+                    u32* dst = (u32*)(Kt + (size_t)jj * DP + (size_t)v * VE);
+                    dst[0] = u.x; dst[1] = u.y; dst[2] = u.z; dst[3] = u.w;
+                }
+            } else {
+                for (int idx = tid; idx < KT * D; idx += 256) {
+                    const int jj = idx / D, d = idx - jj * D;
+                    T v = (T)0;
+                    if (jj < cnt) {
+                        const int t = lo + base + jj;
+                        v = cache[((size_t)pt[t / ps] * ps + t % ps) * (size_t)D + d];
+                    }
+                    Kt[(size_t)jj * DP + d] = v;
+                }
+            }
+            __syncthreads();
+            float dot[HPT];
+#pragma unroll
+            for (int i = 0; i < HPT; ++i) dot[i] = 0.f;
+            const T* kr = Kt + (size_t)j * DP;
+            int d = 0;
+            if (quad) {
+                for (; d < D; d += 4) {
+                    float k0, k1, k2, k3;
+                    if (sizeof(T) == 2) {
+                        const u32 a = *(const u32*)(kr + d), b = *(const u32*)(kr + d + 2);
+                        k0 = bflo(a); k1 = bfhi(a); k2 = bflo(b); k3 = bfhi(b);
+                    } else {
+                        k0 = hb_ld(kr + d); k1 = hb_ld(kr + d + 1); k2 = hb_ld(kr + d + 2); k3 = hb_ld(kr + d + 3);
+                    }
+#pragma unroll
+                    for (int i = 0; i < HPT; ++i) {
+                        const float4 q4 = *(const float4*)(qs + (hs + NS * i) * Dq + d);
+                        dot[i] = fmaf(q4.x, k0, dot[i]); dot[i] = fmaf(q4.y, k1, dot[i]);
+                        dot[i] = fmaf(q4.z, k2, dot[i]); dot[i] = fmaf(q4.w, k3, dot[i]);
+                    }
+                }
+            } else {
+                for (; d < D; ++d) {
+                    const float kv = hb_ld(kr + d);
+#pragma unroll
+                    for (int i = 0; i < HPT; ++i) dot[i] = fmaf(qs[(hs + NS * i) * Dq + d], kv, dot[i]);
+                }
+            }
+            const bool valid = j < cnt;
+#pragma unroll
+            for (int i = 0; i < HPT; ++i) {
+                const float sc = valid ? dot[i] * scale : -INFINITY;
+                float mx = sc;
+#pragma unroll
+                for (int o = KT / 2; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                const float mn = fmaxf(m[i], mx);
+                const float alpha = expf(m[i] - mn);
+                const float e = valid ? expf(sc - mn) : 0.f;
+                float sum = e;
+#pragma unroll
+                for (int o = KT / 2; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+                l[i] = l[i] * alpha + sum;
+                m[i] = mn;
+                pw[j * HB_LAT_HG + hs + NS * i] = e;
+                if (j == 0) al[hs + NS * i] = alpha;
+            }
+            __syncthreads();
+            if (2 * tid < R) {
+                const bool two = 2 * tid + 1 < R;
+#pragma unroll
+                for (int h = 0; h < HB_LAT_HG; ++h) { const float a = al[h]; acc[h][0] *= a; acc[h][1] *= a; }
+                for (int jj = 0; jj < cnt; ++jj) {
+                    float v0, v1 = 0.f;
+                    if (sizeof(T) == 2) {
+                        const u32 u = *(const u32*)(Kt + (size_t)jj * DP + 2 * tid);      // (DP is even and > 2 * tid: the pair lies in the row)
+                        v0 = bflo(u); v1 = bfhi(u);
+                    } else {
+                        v0 = hb_ld(Kt + (size_t)jj * DP + 2 * tid);
+                        if (two) v1 = hb_ld(Kt + (size_t)jj * DP + 2 * tid + 1);
+                    }
+#pragma unroll
+                    for (int h4 = 0; h4 < HB_LAT_HG; h4 += 4) {
+                        const float4 p4 = *(const float4*)(pw + jj * HB_LAT_HG + h4);
+                        acc[h4][0] = fmaf(p4.x, v0, acc[h4][0]); acc[h4][1] = fmaf(p4.x, v1, acc[h4][1]);
+                        acc[h4 + 1][0] = fmaf(p4.y, v0, acc[h4 + 1][0]); acc[h4 + 1][1] = fmaf(p4.y, v1, acc[h4 + 1][1]);
+                        acc[h4 + 2][0] = fmaf(p4.z, v0, acc[h4 + 2][0]); acc[h4 + 2][1] = fmaf(p4.z, v1, acc[h4 + 2][1]);
+                        acc[h4 + 3][0] = fmaf(p4.w, v0, acc[h4 + 3][0]); acc[h4 + 3][1] = fmaf(p4.w, v1, acc[h4 + 3][1]);
+                    }
+                }
+            }
+        }
+        if (j == 0)
+#pragma unroll
+            for (int i = 0; i < HPT; ++i) { ml[2 * (hs + NS * i)] = m[i]; ml[2 * (hs + NS * i) + 1] = l[i]; }
+        __syncthreads();
+        if (2 * tid < R) {
+            const bool two = 2 * tid + 1 < R;
+#pragma unroll
+            for (int h = 0; h < HB_LAT_HG; ++h) {
+                if (h >= hg) break;
+                const int hq = h0 + h;
+                if (part) {
+                    float* dst = part + ((size_t)(row * H + hq) * gridDim.y + seg) * (R + 2);
+                    dst[2 * tid] = acc[h][0];
+                    if (two) dst[2 * tid + 1] = acc[h][1];
+                    if (tid == 0) { dst[R] = ml[2 * h]; dst[R + 1] = ml[2 * h + 1]; }
+                } else {
+                    const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
+                    float* dst = out + (size_t)row * ldo + (size_t)hq * R;
+                    dst[2 * tid] = acc[h][0] / ml[2 * h + 1] * gmul;
+                    if (two) dst[2 * tid + 1] = acc[h][1] / ml[2 * h + 1] * gmul;
+                }
+            }
+        }
+    }
+}
+// row length of the key tile in LDS, in elements: 4-byte aligned rows whose stride in 4-byte words is odd (no two of a wave's rows
+// start in the same bank)
+template <typename T> static int hb_lat_dp(int D) {
+    if (sizeof(T) == 4) return D | 1;
+    int dp = (D + 1) & ~1;
+    return (dp / 2) % 2 ? dp : dp + 2;
 }
 
 // ---- routed feed-forward --------------------------------------------------------------------------------------------------
@@ -2186,6 +2362,7 @@ __global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng,
 
 }  // namespace
 
+#define HB_LAT_MAX_SEG 64     // blocks that share the keys of one row in the few-row latent attention
 #define HB_MOE_GEMV_ROWS 8    // steps of at most this many rows run the routed feed-forward entry by entry
 #define HB_SCAN_CHUNK 64       // rows per chunk of the chunked matrix-state scan; steps of more rows take that form
 #define HB_LRU_SEQ_ROWS 64    // steps of at most this many rows run the gated linear recurrent unit token by token
@@ -2212,6 +2389,7 @@ struct vox_hybrid {
     int max_ne = 0, max_top = 0, max_eff = 0, max_experts = 0;
     bool any_shift = false;
     bool attn_big_lds = false;              // the attention kernel was given the right to more than 64 KB of LDS
+    bool lat_big_lds = false;               // the same for the few-row latent attention
 };
 
 static bool hb_is_attn(int kind) { return kind == VOX_MIXER_POOLED_WINDOW_ATTN || kind == VOX_MIXER_CAUSAL_ATTN || kind == VOX_MIXER_LATENT_ATTN; }
@@ -2412,9 +2590,32 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         const int nwv2 = QG * split, dimp = (D + 3) & ~3;
         const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (R + 2) * 4;
         const int max_keys = max_kvlen < window ? max_kvlen : window;
-        const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
-        const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (R + 2) * 4 <= m->attn_ws_bytes;
         const float* gate = m->proj + L.q_rank + D;
+        if (n <= HB_ATTN_SEG_ROWS) {
+            // few rows: a block per (row, key tiles), all heads against the tile in LDS; the tiles of a row spread over up to
+            // HB_LAT_MAX_SEG blocks whose partial results are merged
+            constexpr int KT = hb_lat_tile<T>::KT;
+            const int nchunks = (max_keys + KT - 1) / KT;
+            int cpb = n <= 8 ? 1 : (n <= 16 ? 2 : 4);
+            if ((nchunks + cpb - 1) / cpb > HB_LAT_MAX_SEG) cpb = (nchunks + HB_LAT_MAX_SEG - 1) / HB_LAT_MAX_SEG;
+            const int nseg2 = (nchunks + cpb - 1) / cpb;
+            const bool seg2 = nseg2 > 1;
+            if (seg2 && (size_t)n * H * nseg2 * (R + 2) * 4 > m->attn_ws_bytes) return vox_fail(VOX_ERR_INVALID, "hybrid_step: attention workspace");
+            const int DP = hb_lat_dp<T>(D), Dq = (D + 3) & ~3;
+            const size_t lds2 = (((size_t)KT * DP * sizeof(T) + 15) / 16) * 16 + (size_t)(HB_LAT_HG * Dq + KT * HB_LAT_HG + HB_LAT_HG * 3) * 4;
+            if (lds2 > 64 * 1024 && !m->lat_big_lds) {
+                VOX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_hb_latent_attn_rows<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                m->lat_big_lds = true;
+            }
+            hipLaunchKernelGGL((k_hb_latent_attn_rows<T>), dim3(n, nseg2), dim3(256), lds2, st, qa, (long)n_proj, (const T*)cache, o, (long)n_proj,
+                               io->pos, io->row_req, io->page_table, io->pt_stride, H, R, r, window, ps, L.scale, cpb,
+                               seg2 ? m->attn_ws : (float*)nullptr, gate, (long)n_proj, L.out_scale, DP);
+            if (seg2)
+                hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg2, o, (long)n_proj, io->pos, H, R, window, P, cpb,
+                                   gate, (long)n_proj, L.out_scale, KT);
+        } else {
+        const int nseg = 1;
+        const bool segmented = false;
         if (lds > 64 * 1024 && !m->attn_big_lds) {
             VOX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_hb_attn<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             m->attn_big_lds = true;
@@ -2425,7 +2626,8 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
                            L.out_scale, 1, (long)D);
         if (segmented)
             hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, o, (long)n_proj, io->pos, H, R, window, P,
-                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale);
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64);
+        }
         // every head's weighted latent times its value expansion
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, o, n_proj, (const T*)L.w_uv, nullptr, m->mix, n_mix, n, L.vdim, R,
                            hb_rowmap{nullptr, nullptr, 0, 1, (long)L.vdim * R, (long)R, (long)L.vdim, 0, nullptr, 0.f}, H));
@@ -2474,7 +2676,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
                            gate, (long)n_proj, L.out_scale, G, (long)G * L.vdim);
         if (segmented)
             hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->mix, (long)n_mix, io->pos, H, L.vdim, window, P,
-                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale);
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64);
     }
     return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
 }
@@ -2715,7 +2917,8 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
             const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN, latent = L.kind == VOX_MIXER_LATENT_ATTN;
             const int max_keys = causal || (latent && L.window < 1) ? cfg->max_seq_len
                                  : (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + (latent ? 0 : cfg->max_seq_len / L.pool + 1);
-            const size_t nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+            size_t nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+            if (latent) nseg = (size_t)(max_keys + 31) / 32 < HB_LAT_MAX_SEG ? (size_t)(max_keys + 31) / 32 : HB_LAT_MAX_SEG;
             const size_t b = (size_t)HB_ATTN_SEG_ROWS * L.heads * nseg * ((latent ? L.kv_rank : L.vdim) + 2) * 4;
             if (b > m->attn_ws_bytes) m->attn_ws_bytes = b;
         }
