@@ -1893,15 +1893,46 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
     const int total = (first > 0 ? first / P : 0) + (p - (first > 0 ? first : 0) + 1);
     const int nseg = ((total + chunk - 1) / chunk + seg_chunks - 1) / seg_chunks;
     const float* src = part + (size_t)(row * H + hq) * nseg_grid * (vdim + 2);
+    // lane s of each 64 segments fetches segment s's maximum and sum; the total is added in segment order
     float mm = -INFINITY;
-    for (int s2 = 0; s2 < nseg; ++s2) mm = fmaxf(mm, src[(size_t)s2 * (vdim + 2) + vdim]);
-    float lt = 0.f;
-    for (int s2 = 0; s2 < nseg; ++s2) lt += src[(size_t)s2 * (vdim + 2) + vdim + 1] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
+    for (int s0 = 0; s0 < nseg; s0 += 64) mm = fmaxf(mm, s0 + lane < nseg ? src[(size_t)(s0 + lane) * (vdim + 2) + vdim] : -INFINITY);
+    mm = hb_wave_max(mm);
     const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
-    for (int j = lane; j < vdim; j += 64) {
-        float a = 0.f;
-        for (int s2 = 0; s2 < nseg; ++s2) a += src[(size_t)s2 * (vdim + 2) + j] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
-        out[(size_t)row * ldo + hq * vdim + j] = a / lt * gmul;
+    float lt = 0.f;
+    float acc[HB_MAX_VPL];
+#pragma unroll
+    for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] = 0.f;
+    for (int s0 = 0; s0 < nseg; s0 += 64) {
+        const bool mine = s0 + lane < nseg;
+        const float wmine = mine ? expf(src[(size_t)(s0 + lane) * (vdim + 2) + vdim] - mm) : 0.f;
+        const float lmine = mine ? src[(size_t)(s0 + lane) * (vdim + 2) + vdim + 1] * wmine : 0.f;
+        const int ns = nseg - s0 < 64 ? nseg - s0 : 64;
+        for (int s2 = 0; s2 < ns; s2 += 4) {
+            // four segments' values on their way before the first is used
+            float v[4][HB_MAX_VPL];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float* sp = src + (size_t)(s0 + (s2 + u < ns ? s2 + u : ns - 1)) * (vdim + 2);
+#pragma unroll
+                for (int e = 0; e < HB_MAX_VPL; ++e) {
+                    const int j = lane + e * 64;
+                    v[u][e] = j < vdim ? sp[j] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (s2 + u >= ns) break;
+                const float w = __shfl(wmine, s2 + u, 64);
+                lt += __shfl(lmine, s2 + u, 64);
+#pragma unroll
+                for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] += v[u][e] * w;
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < HB_MAX_VPL; ++e) {
+        const int j = lane + e * 64;
+        if (j < vdim) out[(size_t)row * ldo + hq * vdim + j] = acc[e] / lt * gmul;
     }
 }
 
@@ -1912,13 +1943,18 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
 // all heads of the group.  Heads are taken in groups of 16.  part != NULL: the block leaves an unnormalised partial result per head
 // (k_hb_attn_merge's layout) for its `cpb` tiles; else it covers all keys and writes o / l * sigmoid(gate) * out_scale.
 #define HB_LAT_HG 16
-template <typename T> struct hb_lat_tile { static constexpr int KT = sizeof(T) == 2 ? 64 : 32; };
+// KT keys per tile; NT threads per block: NT / KT thread groups share the 16 heads of a group for the scores (NT <= 16 * KT), and
+// NT / 256 thread groups share them for the weighted sums (every 256 threads cover the value columns two by two)
+template <typename T> struct hb_lat_tile {
+    static constexpr int KT = sizeof(T) == 2 ? 64 : 32;
+    static constexpr int NT = sizeof(T) == 2 ? 1024 : 512;
+};
 template <typename T>
-__global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, long ldq, const T* cache, float* out, long ldo, const int* pos,
+__global__ __launch_bounds__(hb_lat_tile<T>::NT) void k_hb_latent_attn_rows(const float* qa, long ldq, const T* cache, float* out, long ldo, const int* pos,
                                                              const int* row_req, const int* ptab, int pts, int H, int R, int r, int window,
                                                              int ps, float scale, int cpb, float* part, const float* gate, long ldg,
                                                              float out_scale, int DP) {
-    constexpr int KT = hb_lat_tile<T>::KT, NS = 256 / KT, HPT = HB_LAT_HG / NS;
+    constexpr int KT = hb_lat_tile<T>::KT, NT = hb_lat_tile<T>::NT, NS = NT / KT, HPT = HB_LAT_HG / NS, PVH = HB_LAT_HG / (NT / 256);
     extern __shared__ float sm[];
     const int D = R + r, Dq = (D + 3) & ~3;
     T* Kt = (T*)sm;                                                    // [KT][DP]
@@ -1940,33 +1976,66 @@ __global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, lo
     for (int h0 = 0; h0 < H; h0 += HB_LAT_HG) {
         const int hg = H - h0 < HB_LAT_HG ? H - h0 : HB_LAT_HG;
         __syncthreads();
-        for (int i = tid; i < HB_LAT_HG * Dq; i += 256) {
-            const int h = i / Dq, d = i - h * Dq;
-            qs[i] = (h < hg && d < D) ? qa[(size_t)row * ldq + (size_t)(h0 + h) * D + d] : 0.f;
+        const float* qrow = qa + (size_t)row * ldq + (size_t)h0 * D;
+        if (quad && (ldq % 4 == 0) && ((((size_t)qa) & 15) == 0)) {
+            // the group's queries are one contiguous run of hg * D floats (Dq = D): 16-byte requests, several in flight per thread
+            const int nv = HB_LAT_HG * D / 4, have = hg * D / 4;
+            constexpr int U = 5;
+            for (int i0 = tid; i0 < nv; i0 += NT * U) {
+                float4 u[U];
+#pragma unroll
+                for (int k = 0; k < U; ++k) {
+                    const int idx = i0 + NT * k;
+                    u[k] = idx < have ? *(const float4*)(qrow + 4 * (size_t)idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int k = 0; k < U; ++k) {
+                    const int idx = i0 + NT * k;
+                    if (idx < nv) *(float4*)(qs + 4 * (size_t)idx) = u[k];
+                }
+            }
+        } else {
+            for (int i = tid; i < HB_LAT_HG * Dq; i += NT) {
+                const int h = i / Dq, d = i - h * Dq;
+                qs[i] = (h < hg && d < D) ? qrow[(size_t)h * D + d] : 0.f;
+            }
         }
-        float m[HPT], l[HPT], acc[HB_LAT_HG][2];
+        float m[HPT], l[HPT], acc[PVH][2];
+        const int ct = tid & 255, hb = (tid >> 8) * PVH;      // the thread's column pair (2 ct, 2 ct + 1) and first head of the weighted sums
 #pragma unroll
         for (int i = 0; i < HPT; ++i) { m[i] = -INFINITY; l[i] = 0.f; }
 #pragma unroll
-        for (int h = 0; h < HB_LAT_HG; ++h) acc[h][0] = acc[h][1] = 0.f;
+        for (int h = 0; h < PVH; ++h) acc[h][0] = acc[h][1] = 0.f;
         for (int c = c0; c < c1; ++c) {
             const int base = c * KT, cnt = total - base < KT ? total - base : KT;
             __syncthreads();
             // the tile: key jj of the tile is the token at position lo + base + jj; rows behind the last key are zero
             if (vec) {
-                const int per = D / VE;
-                for (int idx = tid; idx < KT * per; idx += 256) {
-                    const int jj = idx / per, v = idx - jj * per;
-                    uint4 u = make_uint4(0, 0, 0, 0);
-                    if (jj < cnt) {
-                        const int t = lo + base + jj;
-                        u = *(const uint4*)(cache + ((size_t)pt[t / ps] * ps + t % ps) * (size_t)D + (size_t)v * VE);
+                // 16-byte requests, six in flight per thread before the first is stored
+                const int per = D / VE, nv = KT * per;
+                constexpr int U = 6;
+                for (int i0 = tid; i0 < nv; i0 += NT * U) {
+                    uint4 u[U];
+#pragma unroll
+                    for (int k = 0; k < U; ++k) {
+                        const int idx = i0 + NT * k, jj = idx / per, v = idx - jj * per;
+                        u[k] = make_uint4(0, 0, 0, 0);
+                        if (idx < nv && jj < cnt) {
+                            const int t = lo + base + jj;
+                            u[k] = *(const uint4*)(cache + ((size_t)pt[t / ps] * ps + t % ps) * (size_t)D + (size_t)v * VE);
+                        }
                     }
-                    u32* dst = (u32*)(Kt + (size_t)jj * DP + (size_t)v * VE);
-                    dst[0] = u.x; dst[1] = u.y; dst[2] = u.z; dst[3] = u.w;
+#pragma unroll
+                    for (int k = 0; k < U; ++k) {
+                        const int idx = i0 + NT * k, jj = idx / per, v = idx - jj * per;
+                        if (idx < nv) {
+                            u32* dst = (u32*)(Kt + (size_t)jj * DP + (size_t)v * VE);
+                            dst[0] = u[k].x; dst[1] = u[k].y; dst[2] = u[k].z; dst[3] = u[k].w;
+                        }
+                    }
                 }
             } else {
-                for (int idx = tid; idx < KT * D; idx += 256) {
+                for (int idx = tid; idx < KT * D; idx += NT) {
                     const int jj = idx / D, d = idx - jj * D;
                     T v = (T)0;
                     if (jj < cnt) {
@@ -1983,6 +2052,7 @@ __global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, lo
             const T* kr = Kt + (size_t)j * DP;
             int d = 0;
             if (quad) {
+#pragma unroll 4
                 for (; d < D; d += 4) {
                     float k0, k1, k2, k3;
                     if (sizeof(T) == 2) {
@@ -2024,22 +2094,23 @@ __global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, lo
                 if (j == 0) al[hs + NS * i] = alpha;
             }
             __syncthreads();
-            if (2 * tid < R) {
-                const bool two = 2 * tid + 1 < R;
+            if (2 * ct < R) {
+                const bool two = 2 * ct + 1 < R;
 #pragma unroll
-                for (int h = 0; h < HB_LAT_HG; ++h) { const float a = al[h]; acc[h][0] *= a; acc[h][1] *= a; }
+                for (int h = 0; h < PVH; ++h) { const float a = al[hb + h]; acc[h][0] *= a; acc[h][1] *= a; }
+#pragma unroll 4
                 for (int jj = 0; jj < cnt; ++jj) {
                     float v0, v1 = 0.f;
                     if (sizeof(T) == 2) {
-                        const u32 u = *(const u32*)(Kt + (size_t)jj * DP + 2 * tid);      // (DP is even and > 2 * tid: the pair lies in the row)
+                        const u32 u = *(const u32*)(Kt + (size_t)jj * DP + 2 * ct);      // (DP is even and > 2 * ct: the pair lies in the row)
                         v0 = bflo(u); v1 = bfhi(u);
                     } else {
-                        v0 = hb_ld(Kt + (size_t)jj * DP + 2 * tid);
-                        if (two) v1 = hb_ld(Kt + (size_t)jj * DP + 2 * tid + 1);
+                        v0 = hb_ld(Kt + (size_t)jj * DP + 2 * ct);
+                        if (two) v1 = hb_ld(Kt + (size_t)jj * DP + 2 * ct + 1);
                     }
 #pragma unroll
-                    for (int h4 = 0; h4 < HB_LAT_HG; h4 += 4) {
-                        const float4 p4 = *(const float4*)(pw + jj * HB_LAT_HG + h4);
+                    for (int h4 = 0; h4 < PVH; h4 += 4) {
+                        const float4 p4 = *(const float4*)(pw + jj * HB_LAT_HG + hb + h4);
                         acc[h4][0] = fmaf(p4.x, v0, acc[h4][0]); acc[h4][1] = fmaf(p4.x, v1, acc[h4][1]);
                         acc[h4 + 1][0] = fmaf(p4.y, v0, acc[h4 + 1][0]); acc[h4 + 1][1] = fmaf(p4.y, v1, acc[h4 + 1][1]);
                         acc[h4 + 2][0] = fmaf(p4.z, v0, acc[h4 + 2][0]); acc[h4 + 2][1] = fmaf(p4.z, v1, acc[h4 + 2][1]);
@@ -2052,22 +2123,22 @@ __global__ __launch_bounds__(256) void k_hb_latent_attn_rows(const float* qa, lo
 #pragma unroll
             for (int i = 0; i < HPT; ++i) { ml[2 * (hs + NS * i)] = m[i]; ml[2 * (hs + NS * i) + 1] = l[i]; }
         __syncthreads();
-        if (2 * tid < R) {
-            const bool two = 2 * tid + 1 < R;
+        if (2 * ct < R) {
+            const bool two = 2 * ct + 1 < R;
 #pragma unroll
-            for (int h = 0; h < HB_LAT_HG; ++h) {
-                if (h >= hg) break;
-                const int hq = h0 + h;
+            for (int h = 0; h < PVH; ++h) {
+                if (hb + h >= hg) break;
+                const int hq = h0 + hb + h;
                 if (part) {
                     float* dst = part + ((size_t)(row * H + hq) * gridDim.y + seg) * (R + 2);
-                    dst[2 * tid] = acc[h][0];
-                    if (two) dst[2 * tid + 1] = acc[h][1];
-                    if (tid == 0) { dst[R] = ml[2 * h]; dst[R + 1] = ml[2 * h + 1]; }
+                    dst[2 * ct] = acc[h][0];
+                    if (two) dst[2 * ct + 1] = acc[h][1];
+                    if (ct == 0) { dst[R] = ml[2 * (hb + h)]; dst[R + 1] = ml[2 * (hb + h) + 1]; }
                 } else {
                     const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
                     float* dst = out + (size_t)row * ldo + (size_t)hq * R;
-                    dst[2 * tid] = acc[h][0] / ml[2 * h + 1] * gmul;
-                    if (two) dst[2 * tid + 1] = acc[h][1] / ml[2 * h + 1] * gmul;
+                    dst[2 * ct] = acc[h][0] / ml[2 * (hb + h) + 1] * gmul;
+                    if (two) dst[2 * ct + 1] = acc[h][1] / ml[2 * (hb + h) + 1] * gmul;
                 }
             }
         }
@@ -2607,7 +2678,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
                 VOX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_hb_latent_attn_rows<T>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
                 m->lat_big_lds = true;
             }
-            hipLaunchKernelGGL((k_hb_latent_attn_rows<T>), dim3(n, nseg2), dim3(256), lds2, st, qa, (long)n_proj, (const T*)cache, o, (long)n_proj,
+            hipLaunchKernelGGL((k_hb_latent_attn_rows<T>), dim3(n, nseg2), dim3(hb_lat_tile<T>::NT), lds2, st, qa, (long)n_proj, (const T*)cache, o, (long)n_proj,
                                io->pos, io->row_req, io->page_table, io->pt_stride, H, R, r, window, ps, L.scale, cpb,
                                seg2 ? m->attn_ws : (float*)nullptr, gate, (long)n_proj, L.out_scale, DP);
             if (seg2)
