@@ -373,6 +373,31 @@ def test_odd_sizes(dtype):
     check(cfg, S, toks, [9, 2, 33, 5], dtype=dtype, quantile=q)
 
 
+@pytest.mark.parametrize("heads,kv_rank,rot_dim,window", [(5, 40, 8, 70), (20, 24, 0, 0), (16, 112, 16, 33), (3, 8, 8, 1)])
+def test_matrix_core_attention_against_the_few_row_form(heads, kv_rank, rot_dim, window):
+    """bf16 engine, cached rows that are multiples of 16 bytes: steps of more than 32 rows take the matrix-core attention (row tiles of
+    four, heads as the columns of every product).  Two requests whose lengths are no multiples of four share one long step; the same
+    tokens in portions of at most 30 rows take the few-row form.  Both round the same operands, so they agree far more closely than
+    either agrees with the float64 oracle (what is left are bf16 roundings that flip where the products are summed in another order); a sharp softmax makes a key that is wrongly masked show."""
+    cfg = D.config([D.latent(heads=heads, dim=8, rot_dim=rot_dim, vdim=12, q_rank=16, kv_rank=kv_rank, window=window, scale=1.0, mlp=D.dense(16))],
+                   width=32, vocab=48)
+    S = D.random_checkpoint(cfg, seed=95, qk_gain=2.0)
+    seqs = {"a": tokens(131, 48, 96), "b": tokens(46, 48, 97)}
+    want = {k: DR.forward(cfg, S, v) for k, v in seqs.items()}
+    d = U.Driver(cfg, S, dtype=torch.bfloat16, pages=64, max_rows=256)
+    try:
+        one = d.feed([("a", seqs["a"][:129]), ("b", seqs["b"][:45])])
+        long_a = torch.cat([one["a"], d.feed([("a", seqs["a"][129:])])["a"]], 0)
+        long_b = torch.cat([one["b"], d.feed([("b", seqs["b"][45:])])["b"]], 0)
+        d.end("a"); d.end("b")
+        few_a = d.run_cut("a", seqs["a"], [30, 30, 30, 30, 11])
+        few_b = d.run_cut("b", seqs["b"], [30, 16])
+    finally:
+        d.close()
+    assert U.rel_err(long_a, few_a.double()) < 6e-3 and U.rel_err(long_b, few_b.double()) < 6e-3
+    assert U.rel_err(long_a, want["a"], 0.95) < BF16_BAR and U.rel_err(long_b, want["b"], 0.95) < BF16_BAR
+
+
 # ---- through the framework's own entry points -----------------------------------------------------------------------------------------
 
 def test_greedy_generation_through_the_scheduler():

@@ -2152,6 +2152,185 @@ template <typename T> static int hb_lat_dp(int D) {
     return (dp / 2) % 2 ? dp : dp + 2;
 }
 
+// ---- latent attention, steps of many rows, bf16 cache: the matrix-core form -------------------------------------------------------
+// A block takes four consecutive rows of one request, one wave per row, and a group of up to 16 heads; the heads are the 16 columns of
+// every product, so all 16 x 16 entries of a tile share the row's window.  Tiles of 64 keys are staged in LDS twice: as the cache
+// holds them (Kt[key][dim]) and the value part transposed (Vt[value column][key]).  Per tile and wave:
+//   S^T[key][head] = sum_dim Kt[key][dim] Q[head][dim]     v_mfma_f32_16x16x32_bf16, A = Kt rows from LDS, B = the row's query in
+//                                                          registers (fp32 split in two bf16 parts, hi + lo: two products)
+//   running softmax per head over the lane's 16 scores and the four lane groups
+//   O^T[col][head] += sum_key Vt[col][key] P[head][key]    A = Vt rows from LDS; B = the weights as they sit in the lanes after the first
+//                                                          product (lane group g holds keys 4g..4g+3 of each 16-key tile: the k index of
+//                                                          the product is laid out to match, so no weight leaves its lane), hi + lo
+// Scores, maxima, sums and weights are fp32; the two-part operands keep 16 bits of mantissa of the queries and weights.
+// Tile t of the launch is found by walking the requests' row counts (ceil(rows / 4) tiles each); blocks beyond the last tile leave.
+#define HB_LM_VLD 72      // keys per row of the transposed value tile (64 + 8: rows 16 bytes apart in banks)
+__device__ __forceinline__ void hb_split_bf16x8(const float* v, uint4& hi, uint4& lo) {
+    float h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = bfround(v[i]);
+    hi = make_uint4(pack_bf2(h[0], h[1]), pack_bf2(h[2], h[3]), pack_bf2(h[4], h[5]), pack_bf2(h[6], h[7]));
+    lo = make_uint4(pack_bf2(v[0] - h[0], v[1] - h[1]), pack_bf2(v[2] - h[2], v[3] - h[3]), pack_bf2(v[4] - h[4], v[5] - h[5]),
+                    pack_bf2(v[6] - h[6], v[7] - h[7]));
+}
+__device__ __forceinline__ hb_f32x4 hb_mfma_bf16(uint4 a, uint4 b, hb_f32x4 c) {
+    union { uint4 u; hb_bf16x8 v; } x, y;
+    x.u = a; y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x.v, y.v, c, 0, 0, 0);
+}
+template <int KS, int CT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void k_hb_latent_attn_mfma(
+    const float* qa, long ldq, const bf16_t* cache, float* out, long ldo, const int* pos, const int* req_rows, int n_req, const int* ptab, int pts,
+    int H, int R, int r, int window, int ps, float scale, const float* gate, long ldg, float out_scale, int ks_n, int ct_n) {
+    extern __shared__ float sm[];
+    const int D = R + r, DPK = ks_n * 32 + 8;
+    bf16_t* Kt = (bf16_t*)sm;                      // [64][DPK]
+    bf16_t* Vt = Kt + 64 * DPK;                    // [ct_n * 16][HB_LM_VLD]
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
+    int t = blockIdx.x, rq = -1, rs = 0, re = 0;
+    for (int q = 0; q < n_req; ++q) {
+        const int a = req_rows[q], b = req_rows[q + 1], nt = (b - a + 3) >> 2;
+        if (t < nt) { rq = q; rs = a + 4 * t; re = b; break; }
+        t -= nt;
+    }
+    if (rq < 0) return;
+    const int nrows = re - rs < 4 ? re - rs : 4;
+    const bool active = wv < nrows;
+    const int row = rs + (active ? wv : 0);
+    const int p0 = pos[rs], pl = pos[rs + nrows - 1], p = pos[row];
+    const int lo_t = p0 - window + 1 > 0 ? p0 - window + 1 : 0, lo_r = p - window + 1 > 0 ? p - window + 1 : 0;
+    const int nchunks = (pl - lo_t + 64) >> 6;
+    const int* pt = ptab + (size_t)rq * pts;
+    const int h0 = blockIdx.y * 16, hg = H - h0 < 16 ? H - h0 : 16;
+    // the row's query: head `col`, dims ks*32 + g*8 .. +8 of every 32-dim step
+    uint4 qh[KS], ql[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = 0.f;
+        const int d0 = ks * 32 + g * 8;
+        if (ks < ks_n && active && col < hg && d0 < D) {
+            const float* src = qa + (size_t)row * ldq + (size_t)(h0 + col) * D + d0;
+            const float4 a = *(const float4*)src, b = *(const float4*)(src + 4);
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        }
+        hb_split_bf16x8(v, qh[ks], ql[ks]);
+    }
+    // value-tile rows behind the last value column are never written again: zero once
+    for (int i = R * HB_LM_VLD + tid; i < ct_n * 16 * HB_LM_VLD; i += 256) Vt[i] = (bf16_t)0;
+    float m = -INFINITY, l = 0.f;
+    hb_f32x4 oacc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) oacc[ct] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int per = D >> 3, pv = ks_n * 4, nv = 64 * pv;
+    for (int c = 0; c < nchunks; ++c) {
+        const int base = lo_t + c * 64, cnt = pl - base + 1 < 64 ? pl - base + 1 : 64;
+        __syncthreads();
+        constexpr int U = 6;
+        for (int i0 = tid; i0 < nv; i0 += 256 * U) {
+            uint4 u[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) {
+                const int idx = i0 + 256 * k, jj = idx / pv, v = idx - jj * pv;
+                u[k] = make_uint4(0, 0, 0, 0);
+                if (idx < nv && jj < cnt && v < per) {
+                    const int tk = base + jj;
+                    u[k] = *(const uint4*)(cache + ((size_t)pt[tk / ps] * ps + tk % ps) * (size_t)D + (size_t)v * 8);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < U; ++k) {
+                const int idx = i0 + 256 * k, jj = idx / pv, v = idx - jj * pv;
+                if (idx < nv) {
+                    *(uint4*)(Kt + (size_t)jj * DPK + v * 8) = u[k];
+                    const u32 w[4] = {u[k].x, u[k].y, u[k].z, u[k].w};
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        if (v * 8 + i < R) Vt[(size_t)(v * 8 + i) * HB_LM_VLD + jj] = (bf16_t)(i & 1 ? w[i >> 1] >> 16 : w[i >> 1] & 0xffffu);
+                }
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        hb_f32x4 st[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) st[kt] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks < ks_n) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    const uint4 a = *(const uint4*)(Kt + (size_t)(kt * 16 + col) * DPK + ks * 32 + g * 8);
+                    st[kt] = hb_mfma_bf16(a, qh[ks], st[kt]);
+                    st[kt] = hb_mfma_bf16(a, ql[ks], st[kt]);
+                }
+            }
+        }
+        // lane (col, g) holds the scores of head `col` against keys base + kt*16 + g*4 + i
+        float sc[4][4], mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = base + kt * 16 + g * 4 + i;
+                sc[kt][i] = (key >= lo_r && key <= p) ? st[kt][i] * scale : -INFINITY;
+                mx = fmaxf(mx, sc[kt][i]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        const float alpha = mn == -INFINITY ? 1.0f : expf(m - mn);
+        float sum = 0.f, pr[4][4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pr[kt][i] = sc[kt][i] == -INFINITY ? 0.f : expf(sc[kt][i] - mn);
+                sum += pr[kt][i];
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * alpha + sum;
+        m = mn;
+        uint4 ph[2], plo[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const float v[8] = {pr[2 * kk][0], pr[2 * kk][1], pr[2 * kk][2], pr[2 * kk][3], pr[2 * kk + 1][0], pr[2 * kk + 1][1], pr[2 * kk + 1][2],
+                                pr[2 * kk + 1][3]};
+            hb_split_bf16x8(v, ph[kk], plo[kk]);
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ct < ct_n) {
+                hb_f32x4 o = oacc[ct];
+                o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+                    const bf16_t* vr = Vt + (size_t)(ct * 16 + col) * HB_LM_VLD + kk * 32 + g * 4;
+                    const uint2 a0 = *(const uint2*)vr, a1 = *(const uint2*)(vr + 16);
+                    const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                    o = hb_mfma_bf16(a, ph[kk], o);
+                    o = hb_mfma_bf16(a, plo[kk], o);
+                }
+                oacc[ct] = o;
+            }
+        }
+    }
+    if (!active || col >= hg) return;
+    const int hq = h0 + col;
+    const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
+    float* dst = out + (size_t)row * ldo + (size_t)hq * R;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+        if (ct < ct_n)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int cc = ct * 16 + g * 4 + i;
+                if (cc < R) dst[cc] = oacc[ct][i] / l * gmul;
+            }
+}
+
 // ---- routed feed-forward --------------------------------------------------------------------------------------------------
 // One block per row: router logits z_j = router[j] . h in fp32 (lane-strided sums over four waves and a butterfly: an order fixed by
 // the width, the same for every step shape), then one wave: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
@@ -2526,6 +2705,31 @@ static bool hb_try_norm_gemv(const vox_hybrid* m, hipStream_t st, int epi, const
     return m->cfg.norm_kind == VOX_NORM_LAYER && hb_try_ln_gemv<T>(st, epi, X, ldx, rows, nw, m->cfg.eps, W, bias, C, N, K);
 }
 
+// The matrix-core latent attention for steps of many rows over a bf16 cache.  false: the shapes do not fit it (rows of the cache that are
+// no multiple of 16 bytes, a latent beyond 512 values or keys beyond 576) and the caller takes the general kernel.
+static bool hb_try_latent_mfma(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const vox_hybrid_layer& L, const bf16_t* cache, const float* qa,
+                               float* o, long ldp, const float* gate, int n, int n_req, int window, int ps) {
+    const int R = L.kv_rank, r = L.rot_dim, D = R + r;
+    if ((D & 7) || R > 512 || D > 576 || (ldp & 3)) return false;
+    const int ks_n = (D + 31) / 32, ct_n = (R + 15) / 16;
+    const size_t lds = (size_t)64 * (ks_n * 32 + 8) * 2 + (size_t)ct_n * 16 * HB_LM_VLD * 2;
+    const dim3 grid((n + 3) / 4 + n_req, (L.heads + 15) / 16), block(256);
+#define HB_LM(KS_, CT_) \
+    do { \
+        if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_hb_latent_attn_mfma<KS_, CT_>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+        hipLaunchKernelGGL((k_hb_latent_attn_mfma<KS_, CT_>), grid, block, lds, st, qa, ldp, cache, o, ldp, io->pos, io->req_rows, n_req, io->page_table, \
+                           io->pt_stride, L.heads, R, r, window, ps, L.scale, gate, ldp, L.out_scale, ks_n, ct_n); \
+    } while (0)
+    if (ks_n <= 10 && ct_n <= 16) HB_LM(10, 16);
+    else if (ct_n <= 16) HB_LM(18, 16);
+    else HB_LM(18, 32);
+#undef HB_LM
+    (void)m;
+    return true;
+}
+static bool hb_try_latent_mfma(vox_hybrid*, hipStream_t, const vox_hybrid_io*, const vox_hybrid_layer&, const float*, const float*, float*, long,
+                               const float*, int, int, int, int) { return false; }
+
 // One mixer: reads the normed rows (hn != NULL) or norms `cur` itself with L.norm1, adds out_scale * mixer(.) to cur.
 template <typename T>
 static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const vox_hybrid_layer& L, void* cache, float* pool, float* state,
@@ -2684,6 +2888,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
             if (seg2)
                 hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg2, o, (long)n_proj, io->pos, H, R, window, P, cpb,
                                    gate, (long)n_proj, L.out_scale, KT);
+        } else if (hb_try_latent_mfma(m, st, io, L, (const T*)cache, qa, o, (long)n_proj, gate, n, n_req, window, ps)) {
         } else {
         const int nseg = 1;
         const bool segmented = false;
