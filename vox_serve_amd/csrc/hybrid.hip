@@ -32,6 +32,13 @@ __device__ __forceinline__ float hb_wave_max(float v) {
     for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
+// sum of v over a block of 256 threads in a fixed order: butterfly per wave, the four wave sums added in wave order
+__device__ __forceinline__ float hb_block_sum256(float v, float* red) {
+    v = hb_wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return ((red[0] + red[1]) + red[2]) + red[3];
+}
 __device__ __forceinline__ float hb_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float hb_logsigmoid(float x) { return fminf(x, 0.0f) - log1pf(expf(-fabsf(x))); }
 
@@ -238,6 +245,42 @@ __global__ __launch_bounds__(256) void k_hb_rms_groups(const float* x, long ldx,
                 y1[(size_t)r * ldy + g * Wg + i] = v * w1[g * Wg + i];
                 if (w2) y2[(size_t)r * ldy + g * Wg + i] = v * w2[g * Wg + i];
             }
+        }
+    }
+}
+
+// The same norm over ONE slice (the whole row), all four waves on it: thread-strided sum of squares, butterfly per wave, the four wave
+// sums added in wave order -- an order fixed by the width.
+__global__ __launch_bounds__(256) void k_hb_rms_row(const float* x, long ldx, const int* rows, const float* w1, float* y1, const float* w2, float* y2,
+                                                    long ldy, int W, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, src = rows ? rows[r] : r, tid = threadIdx.x;
+    const float* xr = x + (size_t)src * ldx;
+    const bool vec = (W % 4 == 0) && (ldx % 4 == 0) && (ldy % 4 == 0) && (((size_t)x | (size_t)y1 | (size_t)w1 | (size_t)y2 | (size_t)w2) & 15) == 0;
+    float ss = 0.f;
+    if (vec) {
+        for (int i = tid * 4; i < W; i += 1024) {
+            const float4 v = *(const float4*)(xr + i);
+            ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+        }
+    } else {
+        for (int i = tid; i < W; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    }
+    const float inv = 1.0f / sqrtf(hb_block_sum256(ss, red) / (float)W + eps);
+    if (vec) {
+        for (int i = tid * 4; i < W; i += 1024) {
+            const float4 v = *(const float4*)(xr + i), a = *(const float4*)(w1 + i);
+            *(float4*)(y1 + (size_t)r * ldy + i) = make_float4(v.x * inv * a.x, v.y * inv * a.y, v.z * inv * a.z, v.w * inv * a.w);
+            if (w2) {
+                const float4 b2 = *(const float4*)(w2 + i);
+                *(float4*)(y2 + (size_t)r * ldy + i) = make_float4(v.x * inv * b2.x, v.y * inv * b2.y, v.z * inv * b2.z, v.w * inv * b2.w);
+            }
+        }
+    } else {
+        for (int i = tid; i < W; i += 256) {
+            const float v = xr[i] * inv;
+            y1[(size_t)r * ldy + i] = v * w1[i];
+            if (w2) y2[(size_t)r * ldy + i] = v * w2[i];
         }
     }
 }
@@ -1021,13 +1064,6 @@ __global__ __launch_bounds__(256) void k_hb_retention_carry(float* ws, float* st
 }
 
 // ---- latent attention: what a row leaves in the cache, and its query ----------------------------------------------------------
-// sum of v over a block of 256 threads in a fixed order: butterfly per wave, the four wave sums added in wave order
-__device__ __forceinline__ float hb_block_sum256(float v, float* red) {
-    v = hb_wave_sum(v);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return ((red[0] + red[1]) + red[2]) + red[3];
-}
 // proj row = [query latent (q_rank) | key / value latent (R) | rotated key part (r) | gate (H) | ...].  Block (row, 0): the query latent
 // is RMS-normed with its weight in place.  Block (row, 1): the key / value latent is RMS-normed with its weight into the row's cache
 // entry [R + r] (engine dtype), followed by the rotated key part (hb_rot_half on its first `rot` dims).
@@ -2184,7 +2220,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     int H, int R, int r, int window, int ps, float scale, const float* gate, long ldg, float out_scale, int ks_n, int ct_n) {
     extern __shared__ float sm[];
     const int D = R + r, DPK = ks_n * 32 + 8;
-    bf16_t* Kt = (bf16_t*)sm;                      // [64][DPK]
+    long* tokoff = (long*)sm;                      // [64] where the tile's keys start in the cache
+    bf16_t* Kt = (bf16_t*)(sm + 128);              // [64][DPK]
     bf16_t* Vt = Kt + 64 * DPK;                    // [ct_n * 16][HB_LM_VLD]
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
     int t = blockIdx.x, rq = -1, rs = 0, re = 0;
@@ -2224,31 +2261,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) oacc[ct] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
     const int per = D >> 3, pv = ks_n * 4, nv = 64 * pv;
+    // idx / pv as a multiplication (exact for idx * pv < 2^32): the tile loop has no integer division
+    const unsigned pv_magic = (unsigned)((0x100000000ull + (unsigned)pv - 1) / (unsigned)pv);
     for (int c = 0; c < nchunks; ++c) {
         const int base = lo_t + c * 64, cnt = pl - base + 1 < 64 ? pl - base + 1 : 64;
         __syncthreads();
-        constexpr int U = 6;
+        if (tid < 64 && tid < cnt) {
+            const int tk = base + tid;
+            tokoff[tid] = ((long)pt[tk / ps] * ps + tk % ps) * (long)D;
+        }
+        __syncthreads();
+        // the tile as the cache holds it: consecutive lanes take consecutive 16-byte pieces of a key's row (whole cache lines per request)
+        constexpr int U = 9;      // requests in flight per thread: a tile of 64 keys x 576 dims is two such rounds
         for (int i0 = tid; i0 < nv; i0 += 256 * U) {
             uint4 u[U];
 #pragma unroll
             for (int k = 0; k < U; ++k) {
-                const int idx = i0 + 256 * k, jj = idx / pv, v = idx - jj * pv;
+                const int idx = i0 + 256 * k, jj = (int)__umulhi((unsigned)idx, pv_magic), v = idx - jj * pv;
                 u[k] = make_uint4(0, 0, 0, 0);
-                if (idx < nv && jj < cnt && v < per) {
-                    const int tk = base + jj;
-                    u[k] = *(const uint4*)(cache + ((size_t)pt[tk / ps] * ps + tk % ps) * (size_t)D + (size_t)v * 8);
-                }
+                if (idx < nv && jj < cnt && v < per) u[k] = *(const uint4*)(cache + tokoff[jj] + v * 8);
             }
 #pragma unroll
             for (int k = 0; k < U; ++k) {
-                const int idx = i0 + 256 * k, jj = idx / pv, v = idx - jj * pv;
-                if (idx < nv) {
-                    *(uint4*)(Kt + (size_t)jj * DPK + v * 8) = u[k];
-                    const u32 w[4] = {u[k].x, u[k].y, u[k].z, u[k].w};
-#pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        if (v * 8 + i < R) Vt[(size_t)(v * 8 + i) * HB_LM_VLD + jj] = (bf16_t)(i & 1 ? w[i >> 1] >> 16 : w[i >> 1] & 0xffffu);
-                }
+                const int idx = i0 + 256 * k, jj = (int)__umulhi((unsigned)idx, pv_magic), v = idx - jj * pv;
+                if (idx < nv) *(uint4*)(Kt + jj * DPK + v * 8) = u[k];
+            }
+        }
+        __syncthreads();
+        // the value part transposed, from LDS to LDS: lane = key, so the four 2-byte stores of a wave each fall into one row of Vt
+        // (stores of consecutive columns of one key would all hit two banks)
+        {
+            const int jj = tid & 63;
+            for (int c4 = (tid >> 6) * 4; c4 < R; c4 += 16) {
+                const uint2 w = *(const uint2*)(Kt + (size_t)jj * DPK + c4);
+                bf16_t* dst = Vt + (size_t)c4 * HB_LM_VLD + jj;
+                dst[0] = (bf16_t)(w.x & 0xffffu);
+                if (c4 + 1 < R) dst[HB_LM_VLD] = (bf16_t)(w.x >> 16);
+                if (c4 + 2 < R) dst[2 * HB_LM_VLD] = (bf16_t)(w.y & 0xffffu);
+                if (c4 + 3 < R) dst[3 * HB_LM_VLD] = (bf16_t)(w.y >> 16);
             }
         }
         __syncthreads();
@@ -2498,6 +2548,8 @@ struct hb_moe_small {
     int top, experts, ff, shared_ff, ld_act;
     float limit, shared_limit, alpha, up_offset;
     int scale_input;        // the routing weight multiplies the expert's input instead of its output
+    const float* shared_bias;   // [2 * shared_ff] gate, then up biases of the shared unit, or NULL
+    int shared_gelu;            // the shared unit's activation is the tanh form of gelu
 };
 // gate / up products + activation of every entry: block (column tile, entry); a wave takes gate row n and up row ff + n of the
 // entry's expert and stores g * sigmoid(alpha g) * (u + 1) with the clamps of that expert.  act row of an entry: ld_act floats.
@@ -2509,6 +2561,8 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
     const T* wg;
     int N;
     float limit, xs = 1.0f;
+    const float* gb = nullptr;
+    int gelu = 0;
     if (slot < q.top) {
         const int e = q.sel[(size_t)row * q.top + slot];
         if (e >= q.experts) return;
@@ -2520,13 +2574,15 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
         wg = shared_gate_up;
         N = q.shared_ff;
         limit = q.shared_limit;
+        gb = q.shared_bias;
+        gelu = q.shared_gelu;
     }
     if (n >= N) return;
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     const float* x = h + (size_t)row * ldh;
     const bool vec = (W % CH == 0) && ((((size_t)wg) & 15) == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0);
     const float g0 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane, xs), u0 = hb_dot_wave<T>(wg + (size_t)(N + n) * W, x, W, vec, lane, xs);
-    if (lane == 0) act[(size_t)entry * q.ld_act + n] = hb_glu(g0, u0, limit, q.alpha, q.up_offset, 0);
+    if (lane == 0) act[(size_t)entry * q.ld_act + n] = hb_glu(g0 + (gb ? gb[n] : 0.f), u0 + (gb ? gb[N + n] : 0.f), limit, q.alpha, q.up_offset, gelu);
 }
 // down products of a row's entries, weighted and added to the residual stream: a wave per (row, output column):
 // x[row][c] += sum_k wgt_k * (identity ? h[row][c] : down_{e_k}[c] . act_k)  +  shared_down[c] . act_shared, k ascending.
@@ -2690,7 +2746,9 @@ static int hb_layer_proj(const vox_hybrid_layer& L) {
 static void hb_norm(const vox_hybrid* m, hipStream_t st, int n, const float* x, long ldx, const int* rows, const float* w1, float* y1,
                     const float* w2, float* y2, long ldy) {
     const vox_hybrid_config& c = m->cfg;
-    if (c.norm_kind == VOX_NORM_RMS_GROUPS) {
+    if (c.norm_kind == VOX_NORM_RMS_GROUPS && c.norm_groups == 1) {
+        hipLaunchKernelGGL(k_hb_rms_row, dim3(n), dim3(256), 0, st, x, ldx, rows, w1, y1, w2, y2, ldy, c.width, c.eps);
+    } else if (c.norm_kind == VOX_NORM_RMS_GROUPS) {
         hipLaunchKernelGGL(k_hb_rms_groups, dim3(n, (c.norm_groups + 3) / 4 < 8 ? (c.norm_groups + 3) / 4 : 8), dim3(256), 0, st, x, ldx, rows, w1, y1,
                            w2, y2, ldy, c.width, c.norm_groups, c.eps);
     } else {
@@ -2712,7 +2770,7 @@ static bool hb_try_latent_mfma(vox_hybrid* m, hipStream_t st, const vox_hybrid_i
     const int R = L.kv_rank, r = L.rot_dim, D = R + r;
     if ((D & 7) || R > 512 || D > 576 || (ldp & 3)) return false;
     const int ks_n = (D + 31) / 32, ct_n = (R + 15) / 16;
-    const size_t lds = (size_t)64 * (ks_n * 32 + 8) * 2 + (size_t)ct_n * 16 * HB_LM_VLD * 2;
+    const size_t lds = 512 + (size_t)64 * (ks_n * 32 + 8) * 2 + (size_t)ct_n * 16 * HB_LM_VLD * 2;
     const dim3 grid((n + 3) / 4 + n_req, (L.heads + 15) / 16), block(256);
 #define HB_LM(KS_, CT_) \
     do { \
@@ -2967,7 +3025,7 @@ static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const 
     if (n <= HB_MOE_GEMV_ROWS) {
         const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;
         const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha, E.up_offset,
-                             E.scale_input};
+                             E.scale_input, nullptr, 0};
         if (maxf > 0 && per > 0 && (E.experts > 0 || E.shared_ff > 0))
             hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
                                (const T*)E.shared_gate_up, m->moe_act, W, q);
@@ -3036,9 +3094,19 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
         } else if (L.ff > 0 && L.ff_kind == VOX_FF_GATED) {
             // down(act(gate h + b) * (up h + b)) + b: gate and up rows in one product, the activation in place behind it
             if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, hf, W, (const T*)L.w_up, L.b_up, m->ff, 2 * L.ff, n, 2 * L.ff, W));
-            hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (L.ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->ff_act, L.ff, INFINITY, 1.0f,
-                               (const int*)nullptr, 0, 0.0f, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0);
+            const float* hd = parallel ? hf : m->h2;
+            if (n == 1) {
+                // one row: gate and up rows of a column by one wave, biases and activation in its epilogue (the routed feed-forward's
+                // kernel with the dense unit in the place of the shared expert and nothing routed); more rows would stream the matrix
+                // once per row
+                const hb_moe_small q{nullptr, nullptr, 0, 0, 0, L.ff, L.ff, INFINITY, INFINITY, 1.0f, 0.0f, 0, L.b_up, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0};
+                hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((L.ff + 3) / 4, n), dim3(256), 0, st, hd, (long)W, (const T*)nullptr, (const T*)L.w_up,
+                                   m->ff_act, W, q);
+            } else {
+                VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, hd, W, (const T*)L.w_up, L.b_up, m->ff, 2 * L.ff, n, 2 * L.ff, W));
+                hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (L.ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->ff_act, L.ff, INFINITY, 1.0f,
+                                   (const int*)nullptr, 0, 0.0f, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0);
+            }
             VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff_act, L.ff, (const T*)L.w_down, L.b_down, cur, ldx, n, W, L.ff));
         } else if (L.ff > 0) {
             if (parallel) {
