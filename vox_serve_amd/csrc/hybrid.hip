@@ -3170,6 +3170,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         else if (L.kind == VOX_MIXER_LATENT_ATTN) {
             if (L.q_rank < 1 || L.kv_rank < 1 || L.rot_dim < 0 || !L.w_uq || !L.w_ukT || !L.w_uv || !L.q_lat_norm || !L.kv_lat_norm) bad = "latent attention: ranks / expansions / norms";
             else if (L.kv_rank > 64 * HB_MAX_VPL) bad = "latent attention: kv_rank above 512";
+            else if (L.kv_rank + L.rot_dim > 768) bad = "latent attention: kv_rank + rot_dim above 768 (a key tile and 16 queries have to fit the LDS)";
             else if (L.rot_dims < 0 || L.rot_dims > L.rot_dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)) bad = "latent attention: rot_dims";
             else if (L.window < 0) bad = "latent attention: window";
         }
