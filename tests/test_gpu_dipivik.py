@@ -373,10 +373,12 @@ def test_odd_sizes(dtype):
     check(cfg, S, toks, [9, 2, 33, 5], dtype=dtype, quantile=q)
 
 
-@pytest.mark.parametrize("heads,kv_rank,rot_dim,window", [(5, 40, 8, 70), (20, 24, 0, 0), (16, 112, 16, 33), (3, 8, 8, 1)])
+@pytest.mark.parametrize("heads,kv_rank,rot_dim,window", [(5, 40, 8, 70), (20, 24, 0, 0), (16, 112, 16, 33), (3, 8, 8, 1), (2, 200, 136, 50),
+                                                          (2, 272, 64, 90)])
 def test_matrix_core_attention_against_the_few_row_form(heads, kv_rank, rot_dim, window):
     """bf16 engine, cached rows that are multiples of 16 bytes: steps of more than 32 rows take the matrix-core attention (row tiles of
-    four, heads as the columns of every product).  Two requests whose lengths are no multiples of four share one long step; the same
+    four, heads as the columns of every product; the last two cases have more than 320 key dims, the last more than 256 value columns:
+    the kernel's larger register layouts).  Two requests whose lengths are no multiples of four share one long step; the same
     tokens in portions of at most 30 rows take the few-row form.  Both round the same operands, so they agree far more closely than
     either agrees with the float64 oracle (what is left are bf16 roundings that flip where the products are summed in another order); a sharp softmax makes a key that is wrongly masked show."""
     cfg = D.config([D.latent(heads=heads, dim=8, rot_dim=rot_dim, vdim=12, q_rank=16, kv_rank=kv_rank, window=window, scale=1.0, mlp=D.dense(16))],
