@@ -355,9 +355,10 @@ int vox_lm_prefill(vox_lm* m, void* stream, const vox_lm_io* io, const int32_t* 
 
 /* ---- hybrid-mixer LM engine ---------------------------------------------------------------------------------
  * A decoder whose layers mix tokens with a linear recurrence (HGRN2, mLSTM, a real-gated diagonal unit behind a short
- * convolution, a matrix state with token shift and per-channel decay) or with attention over a paged cache (a sliding
- * window that also keeps one mean key / value per block of older tokens, or plain causal attention with normed q / k /
- * v); two mixers may run side by side on the same input; a contiguous range of layers may run several times with the
+ * convolution, a matrix state with token shift and per-channel decay, retention, the gated delta rule) or with attention
+ * over a paged cache (a sliding window that also keeps one mean key / value per block of older tokens, plain causal
+ * attention with normed q / k / v, or attention over a cached low-rank latent); two mixers may run side by side on the
+ * same input; a layer's outputs may carry a layer scale; a contiguous range of layers may run several times with the
  * same weights (every run owns its cache or state).  A layer is sequential (x += mixer(norm1 x); x += ff(norm2 x)) or
  * parallel (x += mixer(norm1 x) + ff(norm2 x)); the feed-forward is dense or a routed mixture of experts.  Residual
  * stream, norms, rotary angles, scores, routers, gates and recurrent states are fp32 in both dtypes; the dtype is the
@@ -365,14 +366,16 @@ int vox_lm_prefill(vox_lm* m, void* stream, const vox_lm_io* io, const int32_t* 
  * (prompt portions next to single decoded tokens); rows of a request are contiguous and ascending in position.      */
 typedef struct vox_hybrid vox_hybrid;
 enum { VOX_MIXER_HGRN2 = 0, VOX_MIXER_POOLED_WINDOW_ATTN = 1, VOX_MIXER_MLSTM = 2, VOX_MIXER_RGLRU = 3, VOX_MIXER_CAUSAL_ATTN = 4,
-       VOX_MIXER_SHIFT_DECAY = 5, VOX_MIXER_LATENT_ATTN = 6, VOX_MIXER_RETENTION = 7 };
+       VOX_MIXER_SHIFT_DECAY = 5, VOX_MIXER_LATENT_ATTN = 6, VOX_MIXER_RETENTION = 7, VOX_MIXER_DELTA = 8 };
 enum { VOX_HYBRID_BF16 = 0, VOX_HYBRID_F32 = 1 };
 enum { VOX_NORM_LAYER = 0 /* weight-only layer norm */, VOX_NORM_RMS_GROUPS = 1 /* RMS norm over norm_groups equal slices */ };
 /* sequential: x += mixer(norm1 x); x += ff(norm2 x).  parallel: x += mixer(norm1 x) + ff(norm2 x).  parallel, one norm:
  * x += mixer(n) + ff(n) with n = norm1 x (norm2 is not used) */
 enum { VOX_BLOCK_SEQUENTIAL = 0, VOX_BLOCK_PARALLEL = 1, VOX_BLOCK_PARALLEL_ONE_NORM = 2 };
 enum { VOX_FF_UP_DOWN = 0 /* down(gelu_erf(up h)) */, VOX_FF_GATED = 1 /* down(act(gate h + b) * (up h + b)) + b */ };
-enum { VOX_ACT_GELU_TANH = 0, VOX_ACT_SWISH = 1 /* g * sigmoid(alpha g) */ };
+enum { VOX_ACT_GELU_TANH = 0, VOX_ACT_SWISH = 1 /* g * sigmoid(alpha g) */, VOX_ACT_RELU2 = 2 /* max(g, 0)^2 */ };
+enum { VOX_EXPERT_GATED = 0 /* down(act(gate h) * (up h + up_offset)), clamped */, VOX_EXPERT_UP_DOWN = 1 /* down(act(up h)) */ };
+enum { VOX_GATE_NONE = 0, VOX_GATE_SIGMOID = 1, VOX_GATE_SILU = 2 };
 enum { VOX_ROUTER_SOFTMAX = 0, VOX_ROUTER_SIGMOID = 1 };
 /* Routed feed-forward.  Router logits z = router . h in fp32; s = softmax(z) over experts + identity outputs; the `top`
  * largest of s + correction are chosen; their weights are s / (sum of the chosen s + 1e-20).  Expert e < experts:
@@ -389,6 +392,11 @@ typedef struct {
     const void* shared_down;      /* [width][shared_ff] */
     int32_t score_kind, renorm, scale_input;
     float up_offset;
+    /* expert_form VOX_EXPERT_UP_DOWN: experts (and the shared one) are down(act(up h)) with act = expert_act (VOX_ACT_RELU2, or
+     * VOX_ACT_SWISH with slope act_alpha); w_gate_up then holds the up rows only, [experts][ff][width] and [shared_ff][width].
+     * router_bias [experts + identity] fp32 or NULL is added to the router logits before the scores are formed. */
+    int32_t expert_form, expert_act;
+    const float* router_bias;
 } vox_hybrid_moe;
 typedef struct {
     int32_t kind, heads, kv_heads, dim, vdim;
@@ -454,6 +462,26 @@ typedef struct {
      * dims, k then times dim^-1/2; S <- decay[h] S + k v^T, o = S^T q; unit RMS per head (weight head_norm [heads*vdim] or none),
      * times silu(gate) */
     const float* decay;                   /* [heads] fp32 */
+    /* layer scale: the mixer's output (ls1) and the feed-forward's (ls2) are multiplied column by column before they join the
+     * residual sum; [width] fp32 or NULL */
+    const float *ls1, *ls2;
+    /* causal attention behind a short convolution (conv_taps >= 1 with conv_w [n_in][conv_taps] fp32, last tap = current token, no
+     * bias): every channel of q | k | v is convolved over time first (the last conv_taps-1 projected rows of a sequence live in the
+     * run's state slot); qk_norm_whole: q and k are RMS-normed over their whole projection (all heads at once) with the weights
+     * q_norm [heads*dim] and k_norm [kv_heads*dim]; then the first rot_dims dims of every head are rotated (interleaved pairs);
+     * sink: one is added to the softmax denominator (a key of score 0 without a value). */
+    int32_t qk_norm_whole, sink;
+    /* gated delta rule (VOX_MIXER_DELTA): w_in rows = q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | beta (heads) | decay
+     * input (lora > 0: the bottleneck, lora rows; else heads rows, or heads*dim with decay_channels) | gate input (gate_rank > 0: the
+     * bottleneck; else heads*vdim).  q | k | v pass a causal convolution (conv_w [2*kv_heads*dim + heads*vdim][conv_taps]) and silu;
+     * q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2; head h reads q / k head h / (heads/kv_heads).
+     * decay g = exp(-exp(a_log[h]) * softplus(d + dt_bias)), d from w_decay2 [rows, lora] when lora > 0; one g per head, or per head and
+     * key channel (decay_channels).  S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Then unit RMS per head over vdim,
+     * times head_norm [vdim], times gate_act (VOX_GATE_*) of the gate (w_gate2 [heads*vdim, gate_rank] when gate_rank > 0).
+     * State of a slot: S [heads][dim][vdim], then the last conv_taps-1 rows of q | k | v before the convolution, oldest first. */
+    int32_t decay_channels, gate_rank, gate_act;
+    const void* w_gate2;
+    const float *a_log, *dt_bias;
 } vox_hybrid_layer;
 typedef struct {
     int32_t layer;       /* index into layers */
@@ -463,7 +491,8 @@ typedef struct {
     float* pool;         /* pooled attention: [max_pages][(page_size-1)/pool+1][kv_heads][dim+vdim] */
     /* HGRN2, retention: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1]; RGLRU: [slots][conv_taps][C] (S, then the last
      * conv_taps-1 inputs of the convolution, oldest first); shift-decay: [slots][heads*dim*dim + width] (S, then the previous
-     * token's normed input) */
+     * token's normed input); delta: [slots][heads*dim*vdim + (conv_taps-1)*n_qkv]; causal attention behind a convolution:
+     * [slots][(conv_taps-1)*n_qkv] beside its cache */
     float* state;
     void* side_cache;    /* the same three for the layer's sibling mixer */
     float* side_pool;
@@ -477,6 +506,7 @@ typedef struct {
     float logit_softcap;                  /* > 0: logits <- cap * tanh(logits / cap) */
     /* bigram_buckets > 0: x0 += bigram[(prev * bigram_mul_prev + id * bigram_mul_cur) mod buckets], row `buckets` for a sequence's first token */
     int32_t bigram_buckets, bigram_mul_prev, bigram_mul_cur;
+    float logit_scale;                    /* logits <- logits * logit_scale (0: as 1) */
 } vox_hybrid_config;
 typedef struct {
     const vox_hybrid_layer* layers;

@@ -1,9 +1,10 @@
 // Hybrid-mixer LM engine: a decoder whose layers mix tokens either with a linear recurrence (HGRN2, mLSTM, a real-gated diagonal
-// unit behind a short convolution, a matrix state with token shift and per-channel decay) or with attention over a paged cache
-// (a sliding window that also keeps one mean key / value per block of older tokens, or plain causal attention with normed
-// q / k / v).  Two mixers may run side by side on one input; a layer is sequential or parallel; its feed-forward is dense or a
-// routed mixture of experts.  A contiguous range of layers may run several times with the same weights; every run owns its
-// cache or recurrent state.
+// unit behind a short convolution, a matrix state with token shift and per-channel decay, retention, the gated delta rule behind
+// short convolutions) or with attention over a paged cache (a sliding window that also keeps one mean key / value per block of
+// older tokens, plain causal attention with normed q / k / v -- optionally behind a short convolution, rotated, with a softmax
+// sink --, or attention over a cached low-rank latent).  Two mixers may run side by side on one input; a layer is sequential or
+// parallel, with an optional layer scale; its feed-forward is dense or a routed mixture of experts.  A contiguous range of layers
+// may run several times with the same weights; every run owns its cache or recurrent state.
 //
 // Numeric rule of this engine: the residual stream, norms, rotary angles, attention scores / softmax, gates, decays and every
 // recurrent state are fp32.  The engine's dtype (bf16 or fp32) is the storage of the large matrices, of the K / V cache and of
@@ -77,13 +78,16 @@ __device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, 
     return hb_wave_sum(a);
 }
 // HB_EPI_SOFTCAP: v <- arg * tanh(v / arg) (arg = the product's hb_rowmap::epi_arg)
-enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3, HB_EPI_SOFTCAP = 4 };
+// HB_EPI_RESID_SCALED: c += v * col_scale[column] (a layer scale; arg = that column's entry); HB_EPI_SCALE: v <- v * arg
+enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3, HB_EPI_SOFTCAP = 4, HB_EPI_RESID_SCALED = 5, HB_EPI_SCALE = 6 };
 template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias, float arg = 0.f) {
     float v = acc + bias;
     if (EPI == HB_EPI_GELU) v = 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
     if (EPI == HB_EPI_TANH) v = tanhf(v);
     if (EPI == HB_EPI_SOFTCAP) v = arg * tanhf(v / arg);
+    if (EPI == HB_EPI_SCALE) v = v * arg;
     if (EPI == HB_EPI_RESID) v = *c + v;
+    if (EPI == HB_EPI_RESID_SCALED) v = *c + v * arg;
     *c = v;
 }
 __device__ __forceinline__ float hb_gelu_tanh(float z) {
@@ -100,8 +104,12 @@ struct hb_rowmap {
     long w_stride, a_stride, c_stride, b_stride;
     const float* a_scale;
     float epi_arg;
+    const float* col_scale;     // HB_EPI_RESID_SCALED: [N] fp32
 };
-static inline hb_rowmap hb_plain() { return hb_rowmap{nullptr, nullptr, 0, 1, 0, 0, 0, 0, nullptr, 0.f}; }
+static inline hb_rowmap hb_plain() { return hb_rowmap{nullptr, nullptr, 0, 1, 0, 0, 0, 0, nullptr, 0.f, nullptr}; }
+template <int EPI> __device__ __forceinline__ float hb_epi_arg(const hb_rowmap& rm, int col) {
+    return EPI == HB_EPI_RESID_SCALED ? rm.col_scale[col] : rm.epi_arg;
+}
 
 // ---- embedding gather: x[row] = table[id]; the second half of both residual buffers keeps the embedding output ----------
 // A bigram table (bg.table != NULL) adds row (prev * mul_prev + id * mul_cur) mod buckets, prev being the token before this one in its
@@ -414,7 +422,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int gm = m0 + (mt0 + i) * 16 + (lane >> 4) * 4 + r;
-                if (gm < M) hb_epilogue<EPI>(C + (size_t)(lst ? lst[gm] : gm) * ldc + gn, acc[i][j][r], b, rm.epi_arg);
+                if (gm < M) hb_epilogue<EPI>(C + (size_t)(lst ? lst[gm] : gm) * ldc + gn, acc[i][j][r], b, hb_epi_arg<EPI>(rm, gn));
             }
         }
 }
@@ -483,7 +491,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int gn = n0 + tx * 4 + j;
-            if (gn < N) hb_epilogue<EPI>(C + (size_t)arow[ty * RM + i] * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f, rm.epi_arg);
+            if (gn < N) hb_epilogue<EPI>(C + (size_t)arow[ty * RM + i] * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f, hb_epi_arg<EPI>(rm, gn));
         }
     }
 }
@@ -557,7 +565,7 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
 #pragma unroll
         for (int j = 0; j < HB_GEMV_CPW; ++j) {
             const float sum = hb_wave_sum(acc[m][j]);
-            if (m < M && n0 + j < N && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n0 + j, sum, bias ? bias[n0 + j] : 0.f, rm.epi_arg);
+            if (m < M && n0 + j < N && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n0 + j, sum, bias ? bias[n0 + j] : 0.f, hb_epi_arg<EPI>(rm, n0 + j));
         }
 }
 
@@ -695,7 +703,7 @@ __global__ __launch_bounds__(512) void k_hb_gemm_rows16(const float* A, long lda
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = kb * 4 + r;
-            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((((((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col]) + red[4][row][col]) + red[5][row][col]) + red[6][row][col]) + red[7][row][col], bz, rm.epi_arg);
+            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((((((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col]) + red[4][row][col]) + red[5][row][col]) + red[6][row][col]) + red[7][row][col], bz, hb_epi_arg<EPI>(rm, n0 + col));
         }
     }
 }
@@ -757,6 +765,8 @@ int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const
     if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     if (epi == HB_EPI_TANH) return hb_gemm_epi<T, HB_EPI_TANH>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     if (epi == HB_EPI_SOFTCAP) return hb_gemm_epi<T, HB_EPI_SOFTCAP>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    if (epi == HB_EPI_RESID_SCALED) return hb_gemm_epi<T, HB_EPI_RESID_SCALED>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    if (epi == HB_EPI_SCALE) return hb_gemm_epi<T, HB_EPI_SCALE>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
 }
 
@@ -1258,6 +1268,308 @@ __global__ __launch_bounds__(1024) void k_hb_rglru_scan_chunked(float* proj, lon
         }
 }
 
+// ---- short causal convolution over the channels of a fused projection ----------------------------------------------------------
+// y[p][c] = sum_j w[c][j] * u[p - (taps-1-j)][c], j ascending (oldest input first), no bias; inputs before the step's first row come
+// from the slot's history ([taps-1][C], oldest first: the rows at positions p0-(taps-1) .. p0-1 of a portion that starts at p0),
+// inputs before the sequence are zero (a portion that starts at position 0 never reads the slot).  u = columns [0, C) of proj.
+__device__ __forceinline__ float hb_conv_taps(const float* proj, long ldp, const float* cw, const float* hist, int row, int rs, int p, int p0,
+                                              int c, int C, int taps) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j, q = p - back;
+        if (q < 0) continue;
+        const float v = row - back >= rs ? proj[(size_t)(row - back) * ldp + c] : hist[(size_t)(q - (p0 - (taps - 1))) * C + c];
+        acc = fmaf(cw[(size_t)c * taps + j], v, acc);
+    }
+    return acc;
+}
+// After every row of the step has read its inputs: history entry i <- the input at position (end - (taps-1) + i), from this step's rows
+// or from the old history (ascending i, in place: entry i reads old entry i + rows).  One thread per channel of one request.
+__device__ __forceinline__ void hb_conv_hist_update(const float* proj, long ldp, float* hist, int rs, int re, int p0, int c, int C, int taps) {
+    const int n = re - rs;
+    for (int i = 0; i < taps - 1; ++i) {
+        const int q = p0 + n - (taps - 1) + i;
+        float v = 0.f;
+        if (q >= p0) v = proj[(size_t)(rs + q - p0) * ldp + c];
+        else if (q >= 0) v = hist[(size_t)(i + n) * C + c];
+        hist[(size_t)i * C + c] = v;
+    }
+}
+
+// ---- gated delta rule ----------------------------------------------------------------------------------------------------------------
+// Columns of a projection row (see hb_delta): the fused projection [q | k | v | beta | decay input | gate input], then what the mixer
+// derives from it: decay and gate pre-activations of the bottleneck forms, the convolved q | k | v, the decays, q . k per key head.
+struct hb_delta_layout {
+    int nq, nqkv, off_b, off_din, off_gin, n_in, ndec, off_dec, off_gate, off_c, off_g, off_kq, n_proj;
+};
+__device__ __forceinline__ float hb_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+// First launch, one thread per (row, element): q | k | v through the convolution and silu; decay g = exp(-exp(a_log[h]) *
+// softplus(d + dt_bias)); beta = sigmoid in place.
+__global__ __launch_bounds__(256) void k_hb_delta_conv(float* proj, long ldp, const float* cw, const float* state, long per_slot, long hist_off,
+                                                       const float* a_log, const float* dt_bias, const int* pos, const int* row_req,
+                                                       const int* req_rows, const int* req_state, hb_delta_layout y, int H, int dim, int taps,
+                                                       int decay_channels) {
+    const int row = blockIdx.x, idx = blockIdx.y * 256 + threadIdx.x;
+    float* pr = proj + (size_t)row * ldp;
+    if (idx < y.nqkv) {
+        const int r = row_req[row], rs = req_rows[r];
+        const float* hist = state + (size_t)req_state[r] * per_slot + hist_off;
+        const float a = hb_conv_taps(proj, ldp, cw, hist, row, rs, pos[row], pos[rs], idx, y.nqkv, taps);
+        pr[y.off_c + idx] = a * hb_sigmoid(a);
+    } else if (idx < y.nqkv + y.ndec) {
+        const int i = idx - y.nqkv, hh = decay_channels ? i / dim : i;
+        pr[y.off_g + i] = expf(-expf(a_log[hh]) * hb_softplus(pr[y.off_dec + i] + dt_bias[i]));
+    } else if (idx < y.nqkv + y.ndec + H) {
+        const int h = idx - y.nqkv - y.ndec;
+        pr[y.off_b + h] = hb_sigmoid(pr[y.off_b + h]);
+    }
+}
+// Second launch.  Blocks (row, g < G), two waves: q head g and k head g of the convolved row to unit vectors (x / sqrt(sum x^2 + 1e-6)),
+// q times dim^-1/2, then q . k.  Blocks (row, G + j) of a request's last row: the convolution's history of 128 channels moves on (every
+// row has read it in the first launch).
+__global__ __launch_bounds__(128) void k_hb_delta_unit(float* proj, long ldp, float* state, long per_slot, long hist_off, const int* pos,
+                                                       const int* row_req, const int* req_rows, const int* req_state, hb_delta_layout y, int G,
+                                                       int dim, int taps) {
+    __shared__ float xs[2][HB_SCAN_MAX_WAVES * 64];
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if ((int)blockIdx.y >= G) {
+        const int r = row_req[row], rs = req_rows[r], re = req_rows[r + 1], c = ((int)blockIdx.y - G) * 128 + threadIdx.x;
+        if (row != re - 1 || c >= y.nqkv) return;
+        hb_conv_hist_update(proj, ldp, state + (size_t)req_state[r] * per_slot + hist_off, rs, re, pos[rs], c, y.nqkv, taps);
+        return;
+    }
+    const int g = blockIdx.y;
+    float* pr = proj + (size_t)row * ldp;
+    float* x = pr + y.off_c + (wv ? y.nq : 0) + (size_t)g * dim;
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += 64) ss = fmaf(x[d], x[d], ss);
+    ss = hb_wave_sum(ss);
+    const float inv = (1.0f / sqrtf(ss + 1e-6f)) * (wv ? 1.0f : 1.0f / sqrtf((float)dim));
+    for (int d = lane; d < dim; d += 64) {
+        const float v = x[d] * inv;
+        x[d] = v;
+        xs[wv][d] = v;
+    }
+    __syncthreads();
+    if (wv == 0) {
+        float dot = 0.f;
+        for (int d = lane; d < dim; d += 64) dot = fmaf(xs[0][d], xs[1][d], dot);
+        dot = hb_wave_sum(dot);
+        if (lane == 0) pr[y.off_kq + g] = dot;
+    }
+}
+// Per head: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Block = (request, head, 64 value columns); wave w keeps DPW
+// key dims of the state in registers for the whole portion.  Per token every thread decays its part of the state and forms its share of
+// (g S)^T k and (g S)^T q; the waves' shares are added in wave order; then u is known to every thread, the state takes k u^T, and the
+// output is (g S)^T q + u (k . q), which is S^T q after the write.  The order of every sum depends on (dim, DPW) only.
+// Long portions run the request's rows in chunks of `chunk_len` side by side (the recurrence is linear in S, column by column):
+//   HB_SCAN_WHOLE   the whole portion from the slot's state, outputs and state stored
+//   HB_SCAN_REDUCE  chunk z from a zero state without outputs -> B; and with the identity as state and zero values -> the chunk's
+//                   transition A [dim][dim], stored transposed (value tiles beyond vdim carry the identity's columns)
+//   HB_SCAN_REPLAY  chunk z replayed from its carry (left in the workspace by k_hb_delta_carry), outputs written
+// Workspace entry of chunk k of request r: index rs / chunk_len + r + k, [H][dim * (vdim + dim)] floats: B [dim][vdim], then A^T.
+enum { HB_SCAN_WHOLE = 0, HB_SCAN_REDUCE = 1, HB_SCAN_REPLAY = 2 };
+template <int DPW>
+__global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_delta_scan(const float* proj, long ldp, float* out, long ldo, float* state,
+                                                                          long per_slot, const int* req_rows, const int* req_state,
+                                                                          const int* pos, int H, int G, int dim, int vdim, hb_delta_layout y,
+                                                                          int decay_channels, int TT, int mode, int chunk_len, float* ws,
+                                                                          const float* head_w, int gate_mode, float eps, float out_scale) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    const int nw = blockDim.x >> 6, dpad = nw * DPW;
+    float* qs = sm;                       // [TT][dpad]
+    float* ks = qs + TT * dpad;           // [TT][dpad]
+    float* gs = ks + TT * dpad;           // [TT][dpad]
+    float* vs = gs + TT * dpad;           // [TT][64]
+    float* sc = vs + TT * 64;             // [TT][2]: beta, q . k
+    float* part = sc + TT * 2;            // [2][nw][2][64]
+    const int vt = (vdim + 63) >> 6, at = (dim + 63) >> 6, tiles = mode == HB_SCAN_REDUCE ? vt + at : vt;
+    const int chunk = mode == HB_SCAN_WHOLE ? 0 : blockIdx.z / tiles, tile = mode == HB_SCAN_WHOLE ? blockIdx.z : blockIdx.z % tiles;
+    const bool ident = tile >= vt;        // this block carries columns of the chunk's transition
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int c = (ident ? tile - vt : tile) * 64 + lane, ncol = ident ? dim : vdim;
+    const int d0 = w * DPW, gq = h / (H / G);
+    const int rs0 = req_rows[r], re0 = req_rows[r + 1];
+    const int rs = mode == HB_SCAN_WHOLE ? rs0 : rs0 + chunk * chunk_len;
+    if (rs >= re0) return;
+    const int re = mode == HB_SCAN_WHOLE || rs + chunk_len > re0 ? re0 : rs + chunk_len;
+    const bool ok = c < ncol, fresh = pos[rs0] == 0;
+    const size_t per_ws = (size_t)dim * (vdim + dim);
+    float* St = state + (size_t)req_state[r] * per_slot + (size_t)h * dim * vdim;
+    if (mode != HB_SCAN_WHOLE) St = ws + ((size_t)(rs0 / chunk_len + r + chunk) * H + h) * per_ws + (ident ? (size_t)dim * vdim : 0);
+    const bool load = mode == HB_SCAN_REPLAY || (mode == HB_SCAN_WHOLE && !fresh);
+    float S[DPW];
+#pragma unroll
+    for (int i = 0; i < DPW; ++i) {
+        S[i] = (ok && load && d0 + i < dim) ? St[(size_t)(d0 + i) * ncol + c] : 0.f;
+        if (ident && d0 + i == c && ok) S[i] = 1.f;
+    }
+    int flip = 0;
+    for (int t0 = rs; t0 < re; t0 += TT) {
+        const int nt = re - t0 < TT ? re - t0 : TT;
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nt * dpad; idx += blockDim.x) {
+            const int tt = idx / dpad, d = idx - tt * dpad;
+            float q = 0.f, k = 0.f, g = 0.f;
+            if (d < dim) {
+                const float* p = proj + (size_t)(t0 + tt) * ldp;
+                q = p[y.off_c + gq * dim + d];
+                k = p[y.off_c + y.nq + gq * dim + d];
+                g = p[y.off_g + (decay_channels ? h * dim + d : h)];
+            }
+            qs[idx] = q; ks[idx] = k; gs[idx] = g;
+        }
+        for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
+            const int tt = idx >> 6, cc = tile * 64 + (idx & 63);
+            vs[idx] = !ident && cc < vdim ? proj[(size_t)(t0 + tt) * ldp + y.off_c + 2 * y.nq + h * vdim + cc] : 0.f;
+        }
+        for (int tt = threadIdx.x; tt < nt; tt += blockDim.x) {
+            const float* p = proj + (size_t)(t0 + tt) * ldp;
+            sc[2 * tt] = p[y.off_b + h];
+            sc[2 * tt + 1] = p[y.off_kq + gq];
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = vs[tt * 64 + lane], beta = sc[2 * tt], kq = sc[2 * tt + 1];
+            // the token's factors of this wave's dims, four at a time (every staged array starts on a 16-byte boundary)
+            const float4* qt = (const float4*)(qs + tt * dpad + d0);
+            const float4* kt = (const float4*)(ks + tt * dpad + d0);
+            const float4* gt = (const float4*)(gs + tt * dpad + d0);
+            float kr[DPW];
+            float pk = 0.f, pq = 0.f;
+#pragma unroll
+            for (int i = 0; i < DPW; i += 4) {
+                const float4 g4 = gt[i >> 2], k4 = kt[i >> 2], q4 = qt[i >> 2];
+                kr[i] = k4.x; kr[i + 1] = k4.y; kr[i + 2] = k4.z; kr[i + 3] = k4.w;
+                float sv = g4.x * S[i];
+                S[i] = sv; pk = fmaf(sv, k4.x, pk); pq = fmaf(sv, q4.x, pq);
+                sv = g4.y * S[i + 1];
+                S[i + 1] = sv; pk = fmaf(sv, k4.y, pk); pq = fmaf(sv, q4.y, pq);
+                sv = g4.z * S[i + 2];
+                S[i + 2] = sv; pk = fmaf(sv, k4.z, pk); pq = fmaf(sv, q4.z, pq);
+                sv = g4.w * S[i + 3];
+                S[i + 3] = sv; pk = fmaf(sv, k4.w, pk); pq = fmaf(sv, q4.w, pq);
+            }
+            float* pt = part + flip * nw * 128;
+            pt[w * 128 + lane] = pk;
+            pt[w * 128 + 64 + lane] = pq;
+            __syncthreads();
+            float pred = pt[lane];
+            for (int k2 = 1; k2 < nw; ++k2) pred += pt[k2 * 128 + lane];
+            const float u = beta * (v - pred);
+#pragma unroll
+            for (int i = 0; i < DPW; ++i) S[i] = fmaf(kr[i], u, S[i]);
+            if (w == 0 && mode != HB_SCAN_REDUCE) {
+                float o = 0.f;
+                if (ok) {
+                    float oq = pt[64 + lane];
+                    for (int k2 = 1; k2 < nw; ++k2) oq += pt[k2 * 128 + 64 + lane];
+                    o = fmaf(u, kq, oq);
+                }
+                if (head_w) {
+                    // the block holds the whole head (vdim <= 64): unit RMS, the shared weight, the gate and the mixer's scale here
+                    const float inv = 1.0f / sqrtf(hb_wave_sum(o * o) / (float)vdim + eps);
+                    float gm = 1.0f;
+                    if (ok && gate_mode != HB_GATE_NONE) {
+                        const float gv = proj[(size_t)(t0 + tt) * ldp + y.off_gate + h * vdim + c];
+                        gm = gate_mode == HB_GATE_SIGMOID ? hb_sigmoid(gv) : gv * hb_sigmoid(gv);
+                    }
+                    o = o * inv * (ok ? head_w[c] : 0.f) * gm * out_scale;
+                }
+                if (ok) out[(size_t)(t0 + tt) * ldo + h * vdim + c] = o;
+            }
+            flip ^= 1;
+        }
+    }
+    if (mode == HB_SCAN_REPLAY) return;
+    if (ok)
+#pragma unroll
+        for (int i = 0; i < DPW; ++i)
+            if (d0 + i < dim) St[ident ? (size_t)c * dim + d0 + i : (size_t)(d0 + i) * ncol + c] = S[i];
+}
+// Between the two chunked passes: the slot's state is pushed through the request's chunks in order, S <- A_k S + B_k (A_k [dim][dim]
+// times S [dim][vdim], sums over the key dim in ascending order); every chunk's workspace entry receives its carry-in in place of B_k,
+// the slot the final state.  The columns of S are independent: one block per (request, head, 16 value columns), dim <= 128.  Thread =
+// (key row d, a share of the 16 columns); the block's columns of S live in LDS between the chunks.  A_k is stored transposed, so row e of
+// A_k^T is one coalesced request of the block's threads; the values of the next 32 rows (or of the first rows of A_k+1, which does not
+// depend on the carry) are on their way from memory while the current 32 are multiplied.
+// ROWS = 64 (dim <= 64) or 128: key rows with a thread each; the 256 / ROWS thread groups share the 16 columns.
+#define HB_DC_COLS 16
+template <int ROWS>
+__global__ __launch_bounds__(256) void k_hb_delta_carry(float* ws, float* state, long per_slot, const int* req_rows, const int* req_state,
+                                                        const int* pos, int H, int dim, int vdim, int chunk_len) {
+    constexpr int CPT = HB_DC_COLS / (256 / ROWS), EG = 32;      // columns per thread (4 | 8); rows of A^T per group
+    __shared__ __attribute__((aligned(16))) float cur[2][ROWS * HB_DC_COLS];
+    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const int d = tid % ROWS, c0 = (tid / ROWS) * CPT, cb = blockIdx.z * HB_DC_COLS;
+    const int nc = (re - rs + chunk_len - 1) / chunk_len, ng = (dim + EG - 1) / EG;
+    const bool fresh = pos[rs] == 0, dok = d < dim;
+    const size_t per_ws = (size_t)dim * (vdim + dim);
+    float* St = state + (size_t)req_state[r] * per_slot + (size_t)h * dim * vdim;
+    float* w0 = ws + ((size_t)(rs / chunk_len + r) * H + h) * per_ws;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const int c = cb + c0 + j;
+        cur[0][d * HB_DC_COLS + c0 + j] = (dok && c < vdim && !fresh) ? St[(size_t)d * vdim + c] : 0.f;
+    }
+    float ar[EG];
+    auto fetch = [&](int k, int g) {      // A_k[d][g*EG .. g*EG + EG) from the transposed store (zeros beyond dim)
+        const float* AT = w0 + (size_t)k * H * per_ws + (size_t)dim * vdim;
+#pragma unroll
+        for (int i = 0; i < EG; ++i) {
+            const int e = g * EG + i;
+            ar[i] = (dok && e < dim) ? AT[(size_t)e * dim + d] : 0.f;
+        }
+    };
+    fetch(0, 0);
+    int flip = 0;
+    for (int k = 0; k < nc; ++k) {
+        float* wk = w0 + (size_t)k * H * per_ws;
+        float acc[CPT], bk[CPT];
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = cb + c0 + j;
+            bk[j] = (dok && c < vdim) ? wk[(size_t)d * vdim + c] : 0.f;
+            acc[j] = 0.f;
+        }
+        __syncthreads();                // the carry-in is complete
+        const float* cv0 = cur[flip] + c0;
+        for (int g = 0; g < ng; ++g) {
+            float a[EG];
+#pragma unroll
+            for (int i = 0; i < EG; ++i) a[i] = ar[i];
+            if (g + 1 < ng) fetch(k, g + 1);
+            else if (k + 1 < nc) fetch(k + 1, 0);
+#pragma unroll
+            for (int i = 0; i < EG; ++i) {
+                const int e = g * EG + i < ROWS ? g * EG + i : ROWS - 1;      // (rows beyond dim meet a = 0)
+                const float4 v0 = *(const float4*)(cv0 + e * HB_DC_COLS);
+                acc[0] = fmaf(a[i], v0.x, acc[0]); acc[1] = fmaf(a[i], v0.y, acc[1]); acc[2] = fmaf(a[i], v0.z, acc[2]); acc[3] = fmaf(a[i], v0.w, acc[3]);
+                if (CPT == 8) {
+                    const float4 v1 = *(const float4*)(cv0 + e * HB_DC_COLS + 4);
+                    acc[CPT - 4] = fmaf(a[i], v1.x, acc[CPT - 4]); acc[CPT - 3] = fmaf(a[i], v1.y, acc[CPT - 3]);
+                    acc[CPT - 2] = fmaf(a[i], v1.z, acc[CPT - 2]); acc[CPT - 1] = fmaf(a[i], v1.w, acc[CPT - 1]);
+                }
+            }
+        }
+        // S <- A S + B into the other buffer; the chunk's entry receives its carry-in
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = cb + c0 + j;
+            if (dok && c < vdim) wk[(size_t)d * vdim + c] = cur[flip][d * HB_DC_COLS + c0 + j];
+            cur[flip ^ 1][d * HB_DC_COLS + c0 + j] = acc[j] + bk[j];
+        }
+        flip ^= 1;
+    }
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const int c = cb + c0 + j;
+        if (dok && c < vdim) St[(size_t)d * vdim + c] = cur[flip][d * HB_DC_COLS + c0 + j];
+    }
+}
+
 // ---- matrix-state recurrence with token shift and a data-dependent decay per key channel ------------------------------------
 // mixes[s][row] = h[row] + (h_prev - h[row]) * mu[s], s < 5; h_prev is the previous row of the request, or what the slot keeps
 // behind its matrix state (the previous step's last normed input), or zero at position 0.
@@ -1355,7 +1667,6 @@ __global__ __launch_bounds__(256) void k_hb_shift_gemv(const float* h, long ldh,
 //   mode 2  chunk z replayed from its carry (left in the workspace by the carry kernel), outputs written
 // Workspace entry of chunk k of request r: index rs / chunk_len + r + k (unique: the chunks of the requests before r number at most
 // rs / chunk_len + r), [H][dim*dim + dim] floats each.
-enum { HB_SCAN_WHOLE = 0, HB_SCAN_REDUCE = 1, HB_SCAN_REPLAY = 2 };
 template <int DPW>
 __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(const float* proj, long ldp, float* out, long ldo, const float* bonus,
                                                                                 float* state, long per_slot, const float* h, long ldh, int W,
@@ -1588,6 +1899,82 @@ __global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* c
     }
 }
 
+// The plain causal form behind a short convolution.  proj row = [q (H*dim) | k (G*dim) | v (G*vdim) | convolved q | k | v at off_y |
+// processed q at off_qc | per block of 256 channels its sums of squares over the q and over the k channels at off_ss].
+// First launch, one thread per (row, channel): the convolution (hb_conv_taps; the history is the whole state slot), and the block's
+// share of the two sums of squares (block order fixed by the channel count).
+__global__ __launch_bounds__(256) void k_hb_attn_conv(float* proj, long ldp, const float* cw, const float* state, long per_slot, const int* pos,
+                                                      const int* row_req, const int* req_rows, const int* req_state, int nq, int nk, int C, int taps,
+                                                      int off_y, int off_ss) {
+    __shared__ float red[2][4];
+    const int row = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    float v = 0.f;
+    if (c < C) {
+        const int r = row_req[row], rs = req_rows[r];
+        v = hb_conv_taps(proj, ldp, cw, state + (size_t)req_state[r] * per_slot, row, rs, pos[row], pos[rs], c, C, taps);
+        proj[(size_t)row * ldp + off_y + c] = v;
+    }
+    const float sq = hb_block_sum256(c < nq ? v * v : 0.f, red[0]), sk = hb_block_sum256(c >= nq && c < nq + nk ? v * v : 0.f, red[1]);
+    if (threadIdx.x == 0) {
+        proj[(size_t)row * ldp + off_ss + 2 * blockIdx.y] = sq;
+        proj[(size_t)row * ldp + off_ss + 2 * blockIdx.y + 1] = sk;
+    }
+}
+// Second launch, one wave per (row, head of q | k | v): q and k RMS-normed -- whole: over the entire projection (the blocks' sums added in
+// block order) with weights [H*dim] / [G*dim]; else per head with weights [dim] shared by heads (NULL: none) --, then the first `rot`
+// dims of the head rotated (interleaved pairs).  q goes to off_qc, k and v into the cache.  Blocks (row, H + 2G + j) of a request's
+// last row: the convolution's history of 64 channels moves on.
+template <typename T>
+__global__ __launch_bounds__(64) void k_hb_attn_norm_rot(float* proj, long ldp, T* cache, float* state, long per_slot, const float* q_norm,
+                                                         const float* k_norm, const float* inv_freq, const int* pos, const int* page,
+                                                         const int* slot, const int* row_req, const int* req_rows, const int* req_state, int H,
+                                                         int G, int dim, int vdim, int rot, int taps, int ps, long v_base, float eps, int off_y,
+                                                         int off_qc, int off_ss, int whole) {
+    const int row = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
+    const int nq = H * dim, nk = G * dim, nv = G * vdim, C = nq + nk + nv;
+    if (hb >= H + 2 * G) {
+        const int r = row_req[row], rs = req_rows[r], re = req_rows[r + 1], c = (hb - H - 2 * G) * 64 + lane;
+        if (row != re - 1 || c >= C) return;
+        hb_conv_hist_update(proj, ldp, state + (size_t)req_state[r] * per_slot, rs, re, pos[rs], c, C, taps);
+        return;
+    }
+    const float* yr = proj + (size_t)row * ldp + off_y;
+    const size_t tok = (size_t)page[row] * ps + slot[row];
+    if (hb >= H + G) {
+        const int g = hb - H - G;
+        for (int j = lane; j < vdim; j += 64) hb_st(cache + v_base + tok * (size_t)nv + g * vdim + j, yr[nq + nk + g * vdim + j]);
+        return;
+    }
+    const bool is_q = hb < H;
+    const int c0 = is_q ? hb * dim : nq + (hb - H) * dim;       // the head's first channel
+    float inv;
+    if (whole) {
+        const float* ss = proj + (size_t)row * ldp + off_ss + (is_q ? 0 : 1);
+        float sum = 0.f;
+        for (int b = 0; b < (C + 255) / 256; ++b) sum += ss[2 * b];
+        inv = 1.0f / sqrtf(sum / (float)(is_q ? nq : nk) + eps);
+    } else {
+        float s2 = 0.f;
+        for (int d = lane; d < dim; d += 64) s2 = fmaf(yr[c0 + d], yr[c0 + d], s2);
+        inv = 1.0f / sqrtf(hb_wave_sum(s2) / (float)dim + eps);
+    }
+    const float* nw = is_q ? q_norm : k_norm;
+    const int w0 = whole ? (is_q ? hb * dim : (hb - H) * dim) : 0;
+    const float pf = (float)pos[row];
+    for (int d = lane; d < dim; d += 64) {
+        float v = yr[c0 + d] * inv * (nw ? nw[w0 + d] : 1.0f);
+        if (d < rot) {
+            const int dp = d ^ 1;
+            const float other = yr[c0 + dp] * inv * (nw ? nw[w0 + dp] : 1.0f);
+            float sn, cs;
+            sincosf(pf * inv_freq[d >> 1], &sn, &cs);
+            v = (d & 1) ? fmaf(v, cs, other * sn) : fmaf(v, cs, -(other * sn));
+        }
+        if (is_q) proj[(size_t)row * ldp + off_qc + c0 + d] = v;
+        else hb_st(cache + tok * (size_t)nk + (c0 - nq) + d, v);
+    }
+}
+
 // mean key / value of a block of `P` tokens, taken from the cache as stored, when the row's token closes the block.
 // pool entry of block b sits with the page of the block's last token t: pool[(page(t) * ppp + (t % ps) / P)][G][dim + vdim].
 template <typename T>
@@ -1669,7 +2056,7 @@ template <typename T>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
                           long v_base, float scale, int split, int seg_chunks, float* part, const float* gate, long ldg, float out_scale,
-                          int Gc, long v_ld) {
+                          int Gc, long v_ld, int sink) {
     extern __shared__ float sm[];
     const int QG = H / G, NWV = QG * split;
     const int dimp = (dim + 3) & ~3;
@@ -1679,9 +2066,9 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
     float* mo = qs + QG * dimp;             // [NWV][vdim + 2]: partial output, maximum, sum of each wave
     const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int qh = wv % QG, sp = wv / QG, hq = g * QG + qh;
-    // Gc heads per cached row (Gc = G: one per block row of the grid; Gc = 1 < G: every group of query heads reads the one shared head),
-    // value rows v_ld apart
-    const int gk = g % Gc;
+    // Gc heads per cached row; the grid's G groups of query heads divide evenly over them (Gc = G: one group per cached head; Gc < G:
+    // G / Gc consecutive groups read the same cached head), value rows v_ld apart
+    const int gk = g / (G / Gc);
     const size_t kld = (size_t)Gc * dim;
     const int p = pos[row];
     const int* pt = ptab + (size_t)row_req[row] * pts;
@@ -1888,13 +2275,15 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
     if (lane == 0) { mine[vdim] = m; mine[vdim + 1] = l; }
     __syncthreads();
     if (sp == 0) {
-        float mm = -INFINITY;
+        // sink: a key of score 0 without a value joins the softmax of the whole row (a segmented launch adds it in the merge)
+        float mm = sink && !part ? 0.f : -INFINITY;
         for (int s2 = 0; s2 < split; ++s2) mm = fmaxf(mm, mo[(size_t)(s2 * QG + qh) * (vdim + 2) + vdim]);
         float lt = 0.f;
         for (int s2 = 0; s2 < split; ++s2) {
             const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
             lt += o2[vdim + 1] * expf(o2[vdim] - mm);
         }
+        if (sink && !part) lt += expf(-mm);
         if (part) {
             float* dst = part + ((size_t)(row * H + hq) * gridDim.z + blockIdx.z) * (vdim + 2);
             for (int j = lane; j < vdim; j += 64) {
@@ -1922,7 +2311,8 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
 
 // few-row steps: the segments' partial results of a (row, head), merged in segment order; output gate applied here
 __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, float* out, long ldo, const int* pos, int H, int vdim,
-                                                      int window, int P, int seg_chunks, const float* gate, long ldg, float out_scale, int chunk) {
+                                                      int window, int P, int seg_chunks, const float* gate, long ldg, float out_scale, int chunk,
+                                                      int sink) {
     const int row = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
     const int p = pos[row];
     const int first = p - window + 1;
@@ -1930,7 +2320,7 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
     const int nseg = ((total + chunk - 1) / chunk + seg_chunks - 1) / seg_chunks;
     const float* src = part + (size_t)(row * H + hq) * nseg_grid * (vdim + 2);
     // lane s of each 64 segments fetches segment s's maximum and sum; the total is added in segment order
-    float mm = -INFINITY;
+    float mm = sink ? 0.f : -INFINITY;      // sink: a key of score 0 without a value
     for (int s0 = 0; s0 < nseg; s0 += 64) mm = fmaxf(mm, s0 + lane < nseg ? src[(size_t)(s0 + lane) * (vdim + 2) + vdim] : -INFINITY);
     mm = hb_wave_max(mm);
     const float gmul = (gate ? hb_sigmoid(gate[(size_t)row * ldg + hq]) : 1.0f) * out_scale;
@@ -1965,6 +2355,7 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
             }
         }
     }
+    if (sink) lt += expf(-mm);
 #pragma unroll
     for (int e = 0; e < HB_MAX_VPL; ++e) {
         const int j = lane + e * 64;
@@ -2386,8 +2777,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // the width, the same for every step shape), then one wave: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
 // index wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
 // sigmoid != 0: s_j = sigmoid(z_j) instead of the softmax; renorm == 0: the weights are the chosen s as they are.
+// bias != NULL: added to the logits before the scores are formed.
 __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh, const float* router, const float* corr, int W, int nE, int top,
-                                                       int* sel, float* wgt, int sigmoid, int renorm) {
+                                                       int* sel, float* wgt, int sigmoid, int renorm, const float* bias) {
     extern __shared__ float sm[];
     float* sc = sm;                    // [nE] logits, then scores
     float* ch = sm + nE;               // [nE] choice values
@@ -2446,7 +2838,7 @@ __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh,
     }
     __syncthreads();
     if (wv != 0) return;
-    for (int i = lane; i < nE; i += 64) sc[i] = ((part[i] + part[nE + i]) + part[2 * nE + i]) + part[3 * nE + i];
+    for (int i = lane; i < nE; i += 64) sc[i] = (((part[i] + part[nE + i]) + part[2 * nE + i]) + part[3 * nE + i]) + (bias ? bias[i] : 0.f);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     if (sigmoid) {
@@ -2534,10 +2926,20 @@ __device__ __forceinline__ float hb_glu(float g0, float u0, float limit, float a
     const float g = fminf(g0, limit), u = fminf(fmaxf(u0, -limit), limit);
     return (gelu ? hb_gelu_tanh(g) : g * hb_sigmoid(alpha * g)) * (u + up_offset);
 }
+// the activation of an up / down unit: the square of relu, or g * sigmoid(alpha g)
+__device__ __forceinline__ float hb_unit_act(float g, int relu2, float alpha) {
+    if (relu2) { const float r = fmaxf(g, 0.f); return r * r; }
+    return g * hb_sigmoid(alpha * g);
+}
+// up_down != 0: gu row = [up (ff)] and y = act(up) (relu2 != 0: the square of relu, else g * sigmoid(alpha g)), nothing clamped.
 __global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y, int ff, float limit, float alpha, const int* sel, int experts,
-                                                      float up_offset, int gelu) {
+                                                      float up_offset, int gelu, int up_down, int relu2) {
     const int row = blockIdx.x;
     if (sel && sel[row] >= experts) return;
+    if (up_down) {
+        for (int j = blockIdx.y * 256 + threadIdx.x; j < ff; j += gridDim.y * 256) y[(size_t)row * ff + j] = hb_unit_act(gu[(size_t)row * ff + j], relu2, alpha);
+        return;
+    }
     for (int j = blockIdx.y * 256 + threadIdx.x; j < ff; j += gridDim.y * 256)
         y[(size_t)row * ff + j] = hb_glu(gu[(size_t)row * 2 * ff + j], gu[(size_t)row * 2 * ff + ff + j], limit, alpha, up_offset, gelu);
 }
@@ -2550,6 +2952,8 @@ struct hb_moe_small {
     int scale_input;        // the routing weight multiplies the expert's input instead of its output
     const float* shared_bias;   // [2 * shared_ff] gate, then up biases of the shared unit, or NULL
     int shared_gelu;            // the shared unit's activation is the tanh form of gelu
+    int up_down, relu2;         // units are down(act(up h)): the matrices hold up rows only; act = the square of relu (else swish)
+    const float* out_scale;     // [W] layer scale of what joins the residual sum, or NULL
 };
 // gate / up products + activation of every entry: block (column tile, entry); a wave takes gate row n and up row ff + n of the
 // entry's expert and stores g * sigmoid(alpha g) * (u + 1) with the clamps of that expert.  act row of an entry: ld_act floats.
@@ -2566,7 +2970,7 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
     if (slot < q.top) {
         const int e = q.sel[(size_t)row * q.top + slot];
         if (e >= q.experts) return;
-        wg = w_gate_up + (size_t)e * 2 * q.ff * W;
+        wg = w_gate_up + (size_t)e * (q.up_down ? 1 : 2) * q.ff * W;
         N = q.ff;
         limit = q.limit;
         if (q.scale_input) xs = q.wgt[(size_t)row * q.top + slot];
@@ -2581,6 +2985,11 @@ __global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     const float* x = h + (size_t)row * ldh;
     const bool vec = (W % CH == 0) && ((((size_t)wg) & 15) == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0);
+    if (q.up_down) {
+        const float u1 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane, xs);
+        if (lane == 0) act[(size_t)entry * q.ld_act + n] = hb_unit_act(u1, q.relu2, q.alpha);
+        return;
+    }
     const float g0 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane, xs), u0 = hb_dot_wave<T>(wg + (size_t)(N + n) * W, x, W, vec, lane, xs);
     if (lane == 0) act[(size_t)entry * q.ld_act + n] = hb_glu(g0 + (gb ? gb[n] : 0.f), u0 + (gb ? gb[N + n] : 0.f), limit, q.alpha, q.up_offset, gelu);
 }
@@ -2608,12 +3017,12 @@ __global__ __launch_bounds__(256) void k_hb_moe_down_combine(const float* h, lon
         const bool vec = avec && (q.shared_ff % CH == 0) && ((((size_t)shared_down) & 15) == 0);
         acc += hb_dot_wave<T>(shared_down + (size_t)c * q.shared_ff, act + (size_t)(row * per + q.top) * q.ld_act, q.shared_ff, vec, lane);
     }
-    if (lane == 0) x[(size_t)row * ldx + c] += acc;
+    if (lane == 0) x[(size_t)row * ldx + c] += q.out_scale ? acc * q.out_scale[c] : acc;
 }
 // x[row] += sum_k wgt[row*top + k] * (identity output ? h[row] : expert_out[row*top + k]), k ascending
 // (scale_input: an expert's output enters with weight 1, its input was scaled instead)
 __global__ __launch_bounds__(256) void k_hb_moe_combine(float* x, long ldx, const float* h, long ldh, const float* eo, const int* sel,
-                                                        const float* wgt, int top, int experts, int W, int scale_input) {
+                                                        const float* wgt, int top, int experts, int W, int scale_input, const float* out_scale) {
     const int row = blockIdx.x;
     for (int i = threadIdx.x; i < W; i += 256) {
         float acc = 0.f;
@@ -2622,7 +3031,7 @@ __global__ __launch_bounds__(256) void k_hb_moe_combine(float* x, long ldx, cons
             const bool ident = sel[en] >= experts;
             acc = fmaf(scale_input && !ident ? 1.0f : wgt[en], ident ? h[(size_t)row * ldh + i] : eo[en * W + i], acc);
         }
-        x[(size_t)row * ldx + i] += acc;
+        x[(size_t)row * ldx + i] += out_scale ? acc * out_scale[i] : acc;
     }
 }
 
@@ -2672,6 +3081,8 @@ __global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng,
 #define HB_MOE_GEMV_ROWS 8    // steps of at most this many rows run the routed feed-forward entry by entry
 #define HB_SCAN_CHUNK 64       // rows per chunk of the chunked matrix-state scan; steps of more rows take that form
 #define HB_LRU_SEQ_ROWS 64    // steps of at most this many rows run the gated linear recurrent unit token by token
+#define HB_DELTA_CHUNK 128     // rows per chunk of the chunked delta-rule scan (every chunk costs a dim x dim x vdim product in the carry)
+#define HB_DELTA_CHUNK_DIM 128 // key dims up to which the delta rule's long portions run in chunks (the carry kernel gives every key row a thread)
 
 struct vox_hybrid {
     vox_ctx* ctx;
@@ -2721,6 +3132,45 @@ static int hb_latent_groups(int H) {
         if (H % g == 0 && H / g <= 16) return g;
     return H;
 }
+// Columns of a delta-rule row: the fused projection, then (each part on a 16-byte boundary) the pre-activations of the bottleneck
+// forms, the convolved q | k | v, the decays and q . k per key head.
+static hb_delta_layout hb_delta(const vox_hybrid_layer& L) {
+    hb_delta_layout y;
+    const int nv = L.heads * L.vdim;
+    y.nq = L.kv_heads * L.dim;
+    y.nqkv = 2 * y.nq + nv;
+    y.off_b = y.nqkv;
+    y.off_din = y.off_b + L.heads;
+    y.ndec = L.decay_channels ? L.heads * L.dim : L.heads;
+    y.off_gin = y.off_din + (L.lora > 0 ? L.lora : y.ndec);
+    y.n_in = y.off_gin + (L.gate_rank > 0 ? L.gate_rank : nv);
+    int next = hb_up4(y.n_in);
+    y.off_dec = y.off_din;
+    if (L.lora > 0) { y.off_dec = next; next += hb_up4(y.ndec); }
+    y.off_gate = y.off_gin;
+    if (L.gate_rank > 0) { y.off_gate = next; next += hb_up4(nv); }
+    y.off_c = next; next += hb_up4(y.nqkv);
+    y.off_g = next; next += hb_up4(y.ndec);
+    y.off_kq = next; next += hb_up4(L.kv_heads);
+    y.n_proj = next;
+    return y;
+}
+// a causal attention layer whose q | k | v pass a convolution first
+static bool hb_conv_attn(const vox_hybrid_layer& L) { return L.kind == VOX_MIXER_CAUSAL_ATTN && L.conv_taps > 0; }
+// Columns of such a layer's row behind the fused projection [q | k | v] (C values): the convolved q | k | v, the processed query, and
+// per block of 256 channels the sums of squares over its q and its k channels.
+struct hb_conv_attn_layout {
+    int off_y, off_qc, off_ss, n_proj;
+};
+static hb_conv_attn_layout hb_conv_attn_cols(const vox_hybrid_layer& L) {
+    const int C = L.heads * L.dim + L.kv_heads * (L.dim + L.vdim);
+    hb_conv_attn_layout y;
+    y.off_y = hb_up4(C);
+    y.off_qc = y.off_y + hb_up4(C);
+    y.off_ss = y.off_qc + hb_up4(L.heads * L.dim);
+    y.n_proj = y.off_ss + hb_up4(2 * ((C + 255) / 256));
+    return y;
+}
 // rows of the fused input projection
 static int hb_layer_in(const vox_hybrid_layer& L) {
     switch (L.kind) {
@@ -2732,6 +3182,7 @@ static int hb_layer_in(const vox_hybrid_layer& L) {
         case VOX_MIXER_SHIFT_DECAY: return 4 * L.heads * L.dim + L.lora;
         case VOX_MIXER_LATENT_ATTN: return L.q_rank + L.kv_rank + L.rot_dim + L.heads;
         case VOX_MIXER_RETENTION: return 2 * L.heads * L.dim + 2 * L.heads * L.vdim;
+        case VOX_MIXER_DELTA: return L.kv_heads > 0 ? hb_delta(L).n_in : -1;
     }
     return -1;
 }
@@ -2740,6 +3191,8 @@ static int hb_layer_proj(const vox_hybrid_layer& L) {
     if (L.kind == VOX_MIXER_RGLRU) return 5 * L.heads * L.dim;                           // + conv output, 2 gates
     if (L.kind == VOX_MIXER_SHIFT_DECAY) return 5 * L.heads * L.dim + L.lora;            // + decay pre-activation
     if (L.kind == VOX_MIXER_LATENT_ATTN) return hb_latent(L).n_proj;
+    if (L.kind == VOX_MIXER_DELTA) return hb_delta(L).n_proj;
+    if (hb_conv_attn(L)) return hb_conv_attn_cols(L).n_proj;
     return hb_layer_in(L);
 }
 
@@ -2788,7 +3241,15 @@ static bool hb_try_latent_mfma(vox_hybrid* m, hipStream_t st, const vox_hybrid_i
 static bool hb_try_latent_mfma(vox_hybrid*, hipStream_t, const vox_hybrid_io*, const vox_hybrid_layer&, const float*, const float*, float*, long,
                                const float*, int, int, int, int) { return false; }
 
-// One mixer: reads the normed rows (hn != NULL) or norms `cur` itself with L.norm1, adds out_scale * mixer(.) to cur.
+// cur += (A . W^T + bias) [* scale column by column]
+template <typename T>
+static int hb_gemm_resid(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* cur, long ldx, int n, int N, int K,
+                         const float* scale) {
+    hb_rowmap rm = hb_plain();
+    rm.col_scale = scale;
+    return hb_gemm<T>(st, scale ? HB_EPI_RESID_SCALED : HB_EPI_RESID, A, lda, W, bias, cur, ldx, n, N, K, rm);
+}
+// One mixer: reads the normed rows (hn != NULL) or norms `cur` itself with L.norm1, adds out_scale * mixer(.) [* ls1] to cur.
 template <typename T>
 static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const vox_hybrid_layer& L, void* cache, float* pool, float* state,
                     const float* hn, float* cur, long ldx, int n, int n_req, int max_kvlen) {
@@ -2850,7 +3311,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         if (!fused_norm)
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj, 3 * HD,
                                (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
-        return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
+        return hb_gemm_resid<T>(st, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix, L.ls1);
     }
     if (!hn && !(n == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, nullptr, L.norm1, (const T*)L.w_in, L.b_in, m->proj, n_in, W))) {
         hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, nullptr, nullptr, (long)W);
@@ -2901,6 +3362,48 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         }
         hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj,
                            2 * L.heads * L.dim + L.heads * L.vdim, (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
+    } else if (L.kind == VOX_MIXER_DELTA) {
+        const hb_delta_layout y = hb_delta(L);
+        const int H = L.heads, G = L.kv_heads, nv = H * L.vdim;
+        const long per_slot = (long)H * L.dim * L.vdim + (long)(L.conv_taps - 1) * y.nqkv, hist_off = (long)H * L.dim * L.vdim;
+        if (L.lora > 0)
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + y.off_din, n_proj, (const T*)L.w_decay2, nullptr, m->proj + y.off_dec, n_proj, n, y.ndec, L.lora));
+        if (L.gate_rank > 0)
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + y.off_gin, n_proj, (const T*)L.w_gate2, nullptr, m->proj + y.off_gate, n_proj, n, nv, L.gate_rank));
+        hipLaunchKernelGGL(k_hb_delta_conv, dim3(n, (y.nqkv + y.ndec + H + 255) / 256), dim3(256), 0, st, m->proj, (long)n_proj, L.conv_w, state,
+                           per_slot, hist_off, L.a_log, L.dt_bias, io->pos, io->row_req, io->req_rows, io->req_state, y, H, L.dim, L.conv_taps,
+                           L.decay_channels);
+        hipLaunchKernelGGL(k_hb_delta_unit, dim3(n, G + (L.conv_taps > 1 ? (y.nqkv + 127) / 128 : 0)), dim3(128), 0, st, m->proj, (long)n_proj,
+                           state, per_slot, hist_off, io->pos, io->row_req, io->req_rows, io->req_state, y, G, L.dim, L.conv_taps);
+        const bool chunked = n > HB_DELTA_CHUNK && m->scan_ws && L.dim <= HB_DELTA_CHUNK_DIM;
+        const int gate_mode = L.gate_act == VOX_GATE_SILU ? (int)HB_GATE_SILU : (L.gate_act == VOX_GATE_SIGMOID ? (int)HB_GATE_SIGMOID : (int)HB_GATE_NONE);
+        // few-row steps with heads of at most 64 value columns (one block holds a head): the scan also applies the head norm, the gate
+        // and the scale (per token that is a reduction inside the sequential loop, which long portions leave to a launch of its own)
+        const bool fused_norm = L.vdim <= 64 && n <= HB_MOE_GEMV_ROWS;
+        auto kern = dpw == 16 ? k_hb_delta_scan<16> : (dpw == 32 ? k_hb_delta_scan<32> : k_hb_delta_scan<64>);
+        // three staged arrays per token here: fewer tokens per tile at the widest heads, so that the tile stays within 64 KB of LDS
+        const int tt = 3072 / dpad >= 16 ? 16 : (3072 / dpad >= 1 ? 3072 / dpad : 1);
+        const size_t lds = (size_t)(3 * tt * dpad + tt * 64 + tt * 2 + 2 * nwv * 128) * 4;
+        if (chunked) {
+            // steps of many rows: chunks of HB_DELTA_CHUNK rows side by side (each chunk's transition and offset from the identity and
+            // from zero, the carries pushed through in order, each chunk replayed from its carry)
+            const int nch = (n + HB_DELTA_CHUNK - 1) / HB_DELTA_CHUNK, at = (L.dim + 63) / 64;
+            hipLaunchKernelGGL(kern, dim3(n_req, H, (vt + at) * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, state,
+                               per_slot, io->req_rows, io->req_state, io->pos, H, G, L.dim, L.vdim, y, L.decay_channels, tt, (int)HB_SCAN_REDUCE,
+                               HB_DELTA_CHUNK, m->scan_ws, (const float*)nullptr, 0, c.eps, L.out_scale);
+            hipLaunchKernelGGL(L.dim <= 64 ? k_hb_delta_carry<64> : k_hb_delta_carry<128>, dim3(n_req, H, (L.vdim + HB_DC_COLS - 1) / HB_DC_COLS),
+                               dim3(256), 0, st, m->scan_ws, state, per_slot, io->req_rows, io->req_state, io->pos, H, L.dim, L.vdim, HB_DELTA_CHUNK);
+            hipLaunchKernelGGL(kern, dim3(n_req, H, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, state,
+                               per_slot, io->req_rows, io->req_state, io->pos, H, G, L.dim, L.vdim, y, L.decay_channels, tt, (int)HB_SCAN_REPLAY,
+                               HB_DELTA_CHUNK, m->scan_ws, (const float*)nullptr, 0, c.eps, L.out_scale);
+        } else {
+            hipLaunchKernelGGL(kern, dim3(n_req, H, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, state, per_slot,
+                               io->req_rows, io->req_state, io->pos, H, G, L.dim, L.vdim, y, L.decay_channels, tt, (int)HB_SCAN_WHOLE, 0,
+                               (float*)nullptr, fused_norm ? L.head_norm : (const float*)nullptr, gate_mode, c.eps, L.out_scale);
+        }
+        if (!fused_norm)
+            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, H), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_proj, y.off_gate,
+                               gate_mode, L.vdim, c.eps, L.out_scale);
     } else if (L.kind == VOX_MIXER_LATENT_ATTN) {
         const hb_latent_layout y = hb_latent(L);
         const int H = L.heads, R = L.kv_rank, r = L.rot_dim, D = R + r, dq = L.dim + r;
@@ -2945,7 +3448,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
                                seg2 ? m->attn_ws : (float*)nullptr, gate, (long)n_proj, L.out_scale, DP);
             if (seg2)
                 hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg2, o, (long)n_proj, io->pos, H, R, window, P, cpb,
-                                   gate, (long)n_proj, L.out_scale, KT);
+                                   gate, (long)n_proj, L.out_scale, KT, 0);
         } else if (hb_try_latent_mfma(m, st, io, L, (const T*)cache, qa, o, (long)n_proj, gate, n, n_req, window, ps)) {
         } else {
         const int nseg = 1;
@@ -2957,10 +3460,10 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, qa, (long)n_proj, (const T*)cache,
                            (const float*)nullptr, o, (long)n_proj, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, D, R, window, P, ps, 1,
                            0L, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr, gate, (long)n_proj,
-                           L.out_scale, 1, (long)D);
+                           L.out_scale, 1, (long)D, 0);
         if (segmented)
             hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, o, (long)n_proj, io->pos, H, R, window, P,
-                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64);
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64, 0);
         }
         // every head's weighted latent times its value expansion
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, o, n_proj, (const T*)L.w_uv, nullptr, m->mix, n_mix, n, L.vdim, R,
@@ -2981,14 +3484,33 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
             hipLaunchKernelGGL(k_hb_rglru_scan, dim3(n_req, (C + 63) / 64), dim3(64), 0, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.lam, state,
                                io->req_rows, io->req_state, io->pos, C, bs, L.conv_taps, L.rec_scale, L.out_scale);
     } else {
-        const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN;
-        const int H = L.heads, G = L.kv_heads, QG = H / G;
+        const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN, conv = hb_conv_attn(L);
+        // query heads per block: the whole group of a key / value head, or (groups of more than 16) its largest divisor up to 16
+        int QG = L.heads / L.kv_heads;
+        if (causal)
+            for (int q2 = QG < 16 ? QG : 16; q2 >= 1; --q2)
+                if ((L.heads / L.kv_heads) % q2 == 0) { QG = q2; break; }
+        const int H = L.heads, G = L.kv_heads, GG = H / QG;
         const int window = causal ? c.max_seq_len : L.window, P = causal ? 1 : L.pool;
         const long v_base = (long)c.max_pages * ps * G * L.dim;
         const int ppp = (ps - 1) / P + 1;
         const bool one_row_each = n == n_req;      // decode steps: every block a row closes was filled by earlier steps
         const hb_qkv_opts op = causal ? hb_qkv_opts{L.q_norm, L.k_norm, L.q_temp_coef, L.q_temp_every > 0 ? L.q_temp_every : 1, L.v_unit_rms}
                                       : hb_qkv_opts{nullptr, nullptr, 0.f, 1, 0};
+        const float* qrows = m->proj;
+        if (conv) {
+            const hb_conv_attn_layout y = hb_conv_attn_cols(L);
+            const int C = n_in;
+            const long per_slot = (long)(L.conv_taps - 1) * C;
+            hipLaunchKernelGGL(k_hb_attn_conv, dim3(n, (C + 255) / 256), dim3(256), 0, st, m->proj, (long)n_proj, L.conv_w, state, per_slot, io->pos,
+                               io->row_req, io->req_rows, io->req_state, H * L.dim, G * L.dim, C, L.conv_taps, y.off_y, y.off_ss);
+            hipLaunchKernelGGL((k_hb_attn_norm_rot<T>), dim3(n, H + 2 * G + (L.conv_taps > 1 ? (C + 63) / 64 : 0)), dim3(64), 0, st, m->proj,
+                               (long)n_proj, (T*)cache, state, per_slot, L.q_norm, L.k_norm, L.inv_freq, io->pos, io->page, io->slot, io->row_req,
+                               io->req_rows, io->req_state, H, G, L.dim, L.vdim, L.rot_dims, L.conv_taps, ps, v_base, c.eps, y.off_y, y.off_qc,
+                               y.off_ss, L.qk_norm_whole);
+            const int off_qc = y.off_qc;
+            qrows = m->proj + off_qc;
+        } else
         hipLaunchKernelGGL((k_hb_attn_prep<T>), dim3(n, H + G), dim3(64), 0, st, m->proj, (long)n_proj, (T*)cache, L.inv_freq, io->pos,
                            io->page, io->slot, H, G, L.dim, L.vdim, causal ? 0 : L.rot_dims, ps, v_base, c.eps,
                            one_row_each && !causal ? pool : (float*)nullptr, io->row_req, io->page_table, io->pt_stride, P, ppp, op);
@@ -3004,28 +3526,30 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
         const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (L.vdim + 2) * 4 <= m->attn_ws_bytes;
         const float* gate = causal ? (const float*)nullptr : m->proj + H * L.dim + G * L.dim + G * L.vdim;      // one logit per query head
-        hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, m->proj, (long)n_proj, (const T*)cache,
-                           pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, window,
+        const int sink = causal && L.sink ? 1 : 0;
+        hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, GG, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, qrows, (long)n_proj, (const T*)cache,
+                           pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, GG, L.dim, L.vdim, window,
                            P, ps, ppp, v_base, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr,
-                           gate, (long)n_proj, L.out_scale, G, (long)G * L.vdim);
+                           gate, (long)n_proj, L.out_scale, G, (long)G * L.vdim, sink);
         if (segmented)
             hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->mix, (long)n_mix, io->pos, H, L.vdim, window, P,
-                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64);
+                               HB_ATTN_SEG, gate, (long)n_proj, L.out_scale, 64, sink);
     }
-    return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
+    return hb_gemm_resid<T>(st, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix, L.ls1);
 }
 
 // Routed feed-forward of the normed rows h2, added to cur.  Few rows: one GEMV pair per routed entry; more: the entries are
 // listed per expert and every expert multiplies its own rows in one tile launch.
 template <typename T>
-static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n) {
+static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n, const float* ls) {
     const int W = m->cfg.width, nE = E.experts + E.identity, top = E.top, ne = n * top, ff = E.ff;
+    const int up_down = E.expert_form == VOX_EXPERT_UP_DOWN ? 1 : 0, relu2 = E.expert_act == VOX_ACT_RELU2 ? 1 : 0, nf = up_down ? 1 : 2;
     hipLaunchKernelGGL(k_hb_moe_router, dim3(n), dim3(256), (size_t)(6 * nE + top) * 4, st, h2, (long)W, E.router, E.correction, W, nE, top,
-                       m->moe_sel, m->moe_wgt, E.score_kind == VOX_ROUTER_SIGMOID ? 1 : 0, E.renorm);
+                       m->moe_sel, m->moe_wgt, E.score_kind == VOX_ROUTER_SIGMOID ? 1 : 0, E.renorm, E.router_bias);
     if (n <= HB_MOE_GEMV_ROWS) {
         const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;
         const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha, E.up_offset,
-                             E.scale_input, nullptr, 0};
+                             E.scale_input, nullptr, 0, up_down, relu2, ls};
         if (maxf > 0 && per > 0 && (E.experts > 0 || E.shared_ff > 0))
             hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
                                (const T*)E.shared_gate_up, m->moe_act, W, q);
@@ -3036,22 +3560,22 @@ static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const 
     if (E.experts > 0) {
         const int cap = m->cfg.max_rows;
         hipLaunchKernelGGL(k_hb_moe_group, dim3(E.experts), dim3(256), 0, st, m->moe_sel, ne, cap, m->moe_list, m->moe_count);
-        VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)2 * ff, n, 2 * ff, W,
-                                            hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W, 0, 0, 0,
+        VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)nf * ff, n, nf * ff, W,
+                                            hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)nf * ff * W, 0, 0, 0,
                                                       E.scale_input ? m->moe_wgt : (const float*)nullptr, 0.f}, E.experts));
         hipLaunchKernelGGL(k_hb_glu_clamp, dim3(ne, (ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, ff, E.limit, E.act_alpha,
-                           m->moe_sel, E.experts, E.up_offset, 0);
+                           m->moe_sel, E.experts, E.up_offset, 0, up_down, relu2);
         VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, m->moe_act, (long)ff, (const T*)E.w_down, nullptr, m->moe_out, (long)W, n, W, ff,
                                             hb_rowmap{m->moe_count, m->moe_list, cap, 1, (long)W * ff, 0, 0, 0}, E.experts));
     }
     hipLaunchKernelGGL(k_hb_moe_combine, dim3(n), dim3(256), 0, st, cur, ldx, h2, (long)W, m->moe_out, m->moe_sel, m->moe_wgt, top, E.experts, W,
-                       E.scale_input);
+                       E.scale_input, ls);
     if (E.shared_ff > 0) {
         const int sf = E.shared_ff;
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, h2, W, (const T*)E.shared_gate_up, nullptr, m->ff, 2 * sf, n, 2 * sf, W));
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, h2, W, (const T*)E.shared_gate_up, nullptr, m->ff, nf * sf, n, nf * sf, W));
         hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (sf + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, sf, E.shared_limit, E.act_alpha,
-                           (const int*)nullptr, 0, E.up_offset, 0);
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->moe_act, sf, (const T*)E.shared_down, nullptr, cur, ldx, n, W, sf));
+                           (const int*)nullptr, 0, E.up_offset, 0, up_down, relu2);
+        VOX_TRY(hb_gemm_resid<T>(st, m->moe_act, sf, (const T*)E.shared_down, nullptr, cur, ldx, n, W, sf, ls));
     }
     return VOX_OK;
 }
@@ -3090,7 +3614,7 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             VOX_TRY(hb_mixer<T>(m, st, io, m->layers[L.sibling], run.side_cache, run.side_pool, run.side_state, hn, cur, ldx, n, n_req, max_kvlen));
         if (L.moe) {
             if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
-            VOX_TRY(hb_moe<T>(m, st, *L.moe, hf, cur, ldx, n));
+            VOX_TRY(hb_moe<T>(m, st, *L.moe, hf, cur, ldx, n, L.ls2));
         } else if (L.ff > 0 && L.ff_kind == VOX_FF_GATED) {
             // down(act(gate h + b) * (up h + b)) + b: gate and up rows in one product, the activation in place behind it
             if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
@@ -3099,15 +3623,16 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
                 // one row: gate and up rows of a column by one wave, biases and activation in its epilogue (the routed feed-forward's
                 // kernel with the dense unit in the place of the shared expert and nothing routed); more rows would stream the matrix
                 // once per row
-                const hb_moe_small q{nullptr, nullptr, 0, 0, 0, L.ff, L.ff, INFINITY, INFINITY, 1.0f, 0.0f, 0, L.b_up, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0};
+                const hb_moe_small q{nullptr, nullptr, 0, 0, 0, L.ff, L.ff, INFINITY, INFINITY, 1.0f, 0.0f, 0, L.b_up, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0,
+                                     0, 0, nullptr};
                 hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((L.ff + 3) / 4, n), dim3(256), 0, st, hd, (long)W, (const T*)nullptr, (const T*)L.w_up,
                                    m->ff_act, W, q);
             } else {
                 VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, hd, W, (const T*)L.w_up, L.b_up, m->ff, 2 * L.ff, n, 2 * L.ff, W));
                 hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (L.ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->ff_act, L.ff, INFINITY, 1.0f,
-                                   (const int*)nullptr, 0, 0.0f, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0);
+                                   (const int*)nullptr, 0, 0.0f, L.ff_act == VOX_ACT_GELU_TANH ? 1 : 0, 0, 0);
             }
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff_act, L.ff, (const T*)L.w_down, L.b_down, cur, ldx, n, W, L.ff));
+            VOX_TRY(hb_gemm_resid<T>(st, m->ff_act, L.ff, (const T*)L.w_down, L.b_down, cur, ldx, n, W, L.ff, L.ls2));
         } else if (L.ff > 0) {
             if (parallel) {
                 VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, hf, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
@@ -3115,19 +3640,20 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
                 hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h, nullptr, nullptr, (long)W);
                 VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
             }
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff));
+            VOX_TRY(hb_gemm_resid<T>(st, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff, L.ls2));
         }
         if (io->trace)
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        if (!(n_out == 1 && !(c.logit_softcap > 0.f) &&
+        if (!(n_out == 1 && !(c.logit_softcap > 0.f) && (c.logit_scale == 0.f || c.logit_scale == 1.0f) &&
               hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr, io->logits, c.vocab, W))) {
             hb_norm(m, st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, nullptr, nullptr, (long)W);
+            const bool scaled = c.logit_scale != 0.f && c.logit_scale != 1.0f;
             hb_rowmap rm = hb_plain();
-            rm.epi_arg = c.logit_softcap;
-            VOX_TRY(hb_gemm<T>(st, c.logit_softcap > 0.f ? HB_EPI_SOFTCAP : HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits,
-                               c.vocab, n_out, c.vocab, W, rm));
+            rm.epi_arg = c.logit_softcap > 0.f ? c.logit_softcap : c.logit_scale;
+            VOX_TRY(hb_gemm<T>(st, c.logit_softcap > 0.f ? HB_EPI_SOFTCAP : (scaled ? HB_EPI_SCALE : HB_EPI_STORE), m->hout, W, (const T*)m->w.head,
+                               nullptr, io->logits, c.vocab, n_out, c.vocab, W, rm));
         }
     }
     VOX_HIP(hipGetLastError());
@@ -3142,6 +3668,8 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
     if (cfg->width < 1 || cfg->vocab < 1 || cfg->page_size < 1 || cfg->max_rows < 1 || cfg->max_batch < 1 || cfg->max_out < 1 || cfg->max_seq_len < 1)
         return vox_fail(VOX_ERR_INVALID, "hybrid_create: bad sizes");
     if (cfg->norm_kind != VOX_NORM_LAYER && cfg->norm_kind != VOX_NORM_RMS_GROUPS) return vox_fail(VOX_ERR_INVALID, "hybrid_create: norm kind %d", cfg->norm_kind);
+    if (cfg->logit_softcap > 0.f && cfg->logit_scale != 0.f && cfg->logit_scale != 1.0f)
+        return vox_fail(VOX_ERR_INVALID, "hybrid_create: a logit scale beside a soft cap");
     if (cfg->norm_kind == VOX_NORM_RMS_GROUPS && (cfg->norm_groups < 1 || cfg->width % cfg->norm_groups != 0))
         return vox_fail(VOX_ERR_INVALID, "hybrid_create: %d norm groups do not divide width %d", cfg->norm_groups, cfg->width);
     vox_hybrid* m = new vox_hybrid();
@@ -3174,13 +3702,26 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
             else if (L.rot_dims < 0 || L.rot_dims > L.rot_dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)) bad = "latent attention: rot_dims";
             else if (L.window < 0) bad = "latent attention: window";
         }
-        else if ((L.kind == VOX_MIXER_HGRN2 || L.kind == VOX_MIXER_MLSTM || L.kind == VOX_MIXER_SHIFT_DECAY || L.kind == VOX_MIXER_RETENTION) && L.dim > 64 * HB_SCAN_MAX_WAVES)
+        else if ((L.kind == VOX_MIXER_HGRN2 || L.kind == VOX_MIXER_MLSTM || L.kind == VOX_MIXER_SHIFT_DECAY || L.kind == VOX_MIXER_RETENTION ||
+                  L.kind == VOX_MIXER_DELTA) && L.dim > 64 * HB_SCAN_MAX_WAVES)
             bad = "recurrent dim above 1024";
+        else if (L.kind == VOX_MIXER_DELTA) {
+            if (L.kv_heads < 1 || L.heads % L.kv_heads != 0) bad = "delta: heads / kv_heads";
+            else if (L.conv_taps < 1 || !L.conv_w) bad = "delta: convolution";
+            else if (!L.a_log || !L.dt_bias || !L.head_norm) bad = "delta: a_log / dt_bias / head_norm";
+            else if (L.lora < 0 || (L.lora > 0 && !L.w_decay2)) bad = "delta: decay bottleneck";
+            else if (L.gate_rank < 0 || (L.gate_rank > 0 && !L.w_gate2)) bad = "delta: gate bottleneck";
+            else if (L.gate_act != VOX_GATE_NONE && L.gate_act != VOX_GATE_SIGMOID && L.gate_act != VOX_GATE_SILU) bad = "delta: gate activation";
+        }
         else if (L.kind == VOX_MIXER_RGLRU && (L.dim != L.vdim || L.conv_taps < 1 || !L.conv_w || !L.w_gates || !L.lam)) bad = "rglru needs conv, gates and lam";
         else if (L.kind == VOX_MIXER_SHIFT_DECAY && (L.dim != L.vdim || L.lora < 1 || !L.shift_mu || !L.w_decay2 || !L.decay0 || !L.bonus || !L.head_norm))
             bad = "shift-decay needs mu, decay and bonus tensors";
         else if (hb_is_attn(L.kind) && L.kind != VOX_MIXER_LATENT_ATTN) {
-            if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || L.heads / L.kv_heads > 16) bad = "heads / kv_heads (group of at most 16)";
+            if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || (L.heads / L.kv_heads > 16 && L.kind != VOX_MIXER_CAUSAL_ATTN))
+                bad = "heads / kv_heads (group of at most 16)";
+            else if (hb_conv_attn(L) && (!L.conv_w || (L.qk_norm_whole && (!L.q_norm || !L.k_norm)))) bad = "attention behind a convolution: conv_w / q_norm / k_norm";
+            else if (hb_conv_attn(L) && (L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq))) bad = "rot_dims";
+            else if (hb_conv_attn(L) && (L.q_temp_coef != 0.f || L.v_unit_rms)) bad = "attention behind a convolution: no query temperature / unit values";
             else if (L.dim > 64 * HB_MAX_DPL) bad = "dim above 512";
             else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && (L.window < 1 || L.pool < 1)) bad = "window / pool";
             else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && (L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq))) bad = "rot_dims";
@@ -3188,6 +3729,8 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         if (!bad && L.moe) {
             const vox_hybrid_moe& E = *L.moe;
             if (E.experts < 0 || E.identity < 0 || E.top < 1 || E.top > E.experts + E.identity) bad = "moe: experts / identity / top";
+            else if (E.expert_form != VOX_EXPERT_GATED && E.expert_form != VOX_EXPERT_UP_DOWN) bad = "moe: expert form";
+            else if (E.expert_form == VOX_EXPERT_UP_DOWN && E.expert_act != VOX_ACT_RELU2 && E.expert_act != VOX_ACT_SWISH) bad = "moe: expert activation";
             else if (!E.router || (!L.norm2 && L.block != VOX_BLOCK_PARALLEL_ONE_NORM)) bad = "moe: router or norm2 missing";
             else if (E.score_kind != VOX_ROUTER_SOFTMAX && E.score_kind != VOX_ROUTER_SIGMOID) bad = "moe: score kind";
             else if (E.experts > 0 && (E.ff < 1 || !E.w_gate_up || !E.w_down)) bad = "moe: expert weights";
@@ -3201,6 +3744,10 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         if (L.ff_kind == VOX_FF_GATED && L.ff > m->max_gated) m->max_gated = L.ff;
         if (L.kind == VOX_MIXER_RETENTION) {
             const size_t f = ((size_t)cfg->max_rows / HB_SCAN_CHUNK + cfg->max_batch + 1) * L.heads * ((size_t)L.dim * L.vdim);
+            if (f > m->scan_ws_floats) m->scan_ws_floats = f;
+        }
+        if (L.kind == VOX_MIXER_DELTA && L.dim <= HB_DELTA_CHUNK_DIM) {
+            const size_t f = ((size_t)cfg->max_rows / HB_DELTA_CHUNK + cfg->max_batch + 1) * L.heads * ((size_t)L.dim * (L.vdim + L.dim));
             if (f > m->scan_ws_floats) m->scan_ws_floats = f;
         }
         if (L.kind == VOX_MIXER_SHIFT_DECAY) {
@@ -3224,7 +3771,8 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         if (r.layer < 0 || r.layer >= cfg->n_layers) bad = "layer index";
         else {
             const vox_hybrid_layer& L = m->layers[r.layer];
-            if (hb_is_attn(L.kind) ? (!r.cache || (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.pool)) : !r.state) bad = "missing cache / state";
+            if (hb_is_attn(L.kind) ? (!r.cache || (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.pool) || (hb_conv_attn(L) && L.conv_taps > 1 && !r.state))
+                                   : !r.state) bad = "missing cache / state";
             else if (cfg->bigram_buckets > 0 && (!w->bigram || !w->prev_token)) bad = "bigram table / previous-token state";
             else if (L.sibling >= 0) {
                 const vox_hybrid_layer& S2 = m->layers[L.sibling];

@@ -1,8 +1,10 @@
 """Host side of `vox_hybrid_*`: the engine for decoders that mix tokens with linear recurrences (HGRN2, mLSTM, a real-gated
 diagonal unit behind a short convolution, a matrix state with token shift and per-channel decay, retention with a fixed decay
-per head) and with attention over a paged cache (a sliding window with pooled history, plain causal attention with normed
-q / k / v, or windowed attention whose keys and values are expanded from a cached low-rank latent), optionally two mixers side by
-side, sequential or parallel layers, a dense or a routed feed-forward, and a range of layers looped over shared weights.
+per head, the gated delta rule behind short convolutions) and with attention over a paged cache (a sliding window with pooled
+history, plain causal attention with normed q / k / v -- optionally behind a short convolution, rotated, with a softmax sink --, or
+windowed attention whose keys and values are expanded from a cached low-rank latent), optionally two mixers side by
+side, sequential or parallel layers with an optional layer scale, a dense or a routed feed-forward, and a range of layers looped over
+shared weights.
 
 It reuses the plan / stream / hipGraph machinery of the other LM engines (`Qwen3Engine`): one pinned int32 plan block per
 step, decode steps captured per batch size.  Beyond the K / V pages that the worker hands out, every request holds one
@@ -21,16 +23,18 @@ from . import _native as N
 from .engine import Qwen3Engine
 
 MIXER_HGRN2, MIXER_POOLED_WINDOW_ATTN, MIXER_MLSTM, MIXER_RGLRU, MIXER_CAUSAL_ATTN, MIXER_SHIFT_DECAY = 0, 1, 2, 3, 4, 5
-MIXER_LATENT_ATTN, MIXER_RETENTION = 6, 7
+MIXER_LATENT_ATTN, MIXER_RETENTION, MIXER_DELTA = 6, 7, 8
 MIXER_KINDS = {"hgrn2": MIXER_HGRN2, "attention": MIXER_POOLED_WINDOW_ATTN, "mlstm": MIXER_MLSTM, "rglru": MIXER_RGLRU,
                "causal_attention": MIXER_CAUSAL_ATTN, "shift_decay": MIXER_SHIFT_DECAY, "latent_attention": MIXER_LATENT_ATTN,
-               "retention": MIXER_RETENTION}
+               "retention": MIXER_RETENTION, "delta": MIXER_DELTA}
 ATTENTION_KINDS = ("attention", "causal_attention", "latent_attention")
 NORM_KINDS = {"layer": 0, "rms_groups": 1}
 BLOCK_FORMS = {"sequential": 0, "parallel": 1, "parallel_one_norm": 2}
 FF_KINDS = {"up_down": 0, "gated": 1}
-ACT_KINDS = {"gelu_tanh": 0, "swish": 1}
+ACT_KINDS = {"gelu_tanh": 0, "swish": 1, "relu2": 2}
 ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+EXPERT_FORMS = {"gated": 0, "up_down": 1}
+GATE_KINDS = {"none": 0, "sigmoid": 1, "silu": 2}
 
 
 @dataclass
@@ -48,6 +52,9 @@ class MoECfg:
     renorm: bool = True             # weights divided by the sum of the chosen scores
     scale_input: bool = False       # the weight multiplies what the expert reads, not what it returns
     up_offset: float = 1.0          # y = g * sigmoid(act_alpha g) * (u + up_offset)
+    expert_form: str = "gated"      # "gated" clamped gated units | "up_down" down(act(up h)): experts and the shared one
+    expert_act: str = "swish"       # activation of the up_down form ("relu2" | "swish" with slope act_alpha)
+    router_bias: bool = False       # a bias [experts + identity] is added to the router logits
 
 
 @dataclass
@@ -80,6 +87,12 @@ class MixerCfg:
     kv_rank: int = 0                # latent attention: width of the cached key / value latent
     rot_dim: int = 0                # latent attention: rotated query / key dims per head (the key part is shared by all heads)
     decay: Optional[List[float]] = None     # retention: one decay per head
+    layer_scale: bool = False       # the mixer's and the feed-forward's outputs are multiplied by a vector each (ls1, ls2)
+    qk_norm_whole: bool = False     # causal attention behind a convolution: q / k RMS-normed over the whole projection
+    sink: bool = False              # causal attention: one is added to the softmax denominator
+    decay_channels: bool = False    # delta: one decay per head and key channel (else per head)
+    gate_rank: int = 0              # delta: width of the gate bottleneck (0: one projection); `lora` is the decay bottleneck's
+    gate_act: str = "silu"          # delta: activation of the output gate ("none" | "sigmoid" | "silu")
     side: Optional["MixerCfg"] = None   # a second mixer on the same normed input, added to the same sum
     moe: Optional[MoECfg] = None    # routed feed-forward (instead of the dense one)
 
@@ -95,6 +108,9 @@ class MixerCfg:
             return 2 * h * d
         if self.kind == "causal_attention":
             return h * d + self.kv_heads * (d + v)
+        if self.kind == "delta":
+            nd = h * d if self.decay_channels else h
+            return 2 * self.kv_heads * d + h * v + h + (self.lora or nd) + (self.gate_rank or h * v)
         if self.kind == "shift_decay":
             return 4 * h * d + self.lora
         if self.kind == "latent_attention":
@@ -112,6 +128,10 @@ class MixerCfg:
     def state_floats(self, width: int) -> int:
         """fp32 values of one recurrent-state slot (0 for attention)."""
         h, d, v = self.heads, self.dim, self.vdim
+        if self.kind == "delta":
+            return h * d * v + (self.conv_taps - 1) * (2 * self.kv_heads * d + h * v)
+        if self.kind == "causal_attention":
+            return max(self.conv_taps - 1, 0) * self.n_in         # the convolution's history (0: no state slot)
         return {"hgrn2": h * d * v, "mlstm": h * (d * v + d + 1), "rglru": max(self.conv_taps, 1) * h * d,
                 "shift_decay": h * d * d + width, "retention": h * d * v}.get(self.kind, 0)
 
@@ -128,6 +148,8 @@ class HybridCfg:
     embed_scale: float = 1.0
     logit_softcap: float = 0.0      # > 0: logits <- cap * tanh(logits / cap)
     bigram: Optional[tuple] = None  # (buckets, mul_prev, mul_cur): x0 += bigram[(prev * mul_prev + id * mul_cur) mod buckets]
+    logit_scale: float = 1.0        # logits <- logits * logit_scale
+    norm_one_plus: bool = False     # norm weights are stored around zero: the engine multiplies by 1 + w
 
     def runs(self):
         """[(layer index, loop_in)] in execution order; loop_in marks the first layer of every pass of the looped range."""
@@ -145,7 +167,8 @@ class HybridMoEC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("experts", "identity", "top", "ff", "shared_ff")] + \
                [(n, ctypes.c_float) for n in ("limit", "shared_limit", "act_alpha")] + \
                [(n, ctypes.c_void_p) for n in ("router", "correction", "w_gate_up", "w_down", "shared_gate_up", "shared_down")] + \
-               [(n, ctypes.c_int32) for n in ("score_kind", "renorm", "scale_input")] + [("up_offset", ctypes.c_float)]
+               [(n, ctypes.c_int32) for n in ("score_kind", "renorm", "scale_input")] + [("up_offset", ctypes.c_float)] + \
+               [("expert_form", ctypes.c_int32), ("expert_act", ctypes.c_int32), ("router_bias", ctypes.c_void_p)]
 
 
 class HybridLayerC(ctypes.Structure):
@@ -163,7 +186,10 @@ class HybridLayerC(ctypes.Structure):
                 ("ff_kind", ctypes.c_int32), ("ff_act", ctypes.c_int32), ("b_up", ctypes.c_void_p), ("b_down", ctypes.c_void_p),
                 ("q_rank", ctypes.c_int32), ("kv_rank", ctypes.c_int32), ("rot_dim", ctypes.c_int32),
                 ("w_uq", ctypes.c_void_p), ("w_ukT", ctypes.c_void_p), ("w_uv", ctypes.c_void_p),
-                ("q_lat_norm", ctypes.c_void_p), ("kv_lat_norm", ctypes.c_void_p), ("decay", ctypes.c_void_p)]
+                ("q_lat_norm", ctypes.c_void_p), ("kv_lat_norm", ctypes.c_void_p), ("decay", ctypes.c_void_p),
+                ("ls1", ctypes.c_void_p), ("ls2", ctypes.c_void_p), ("qk_norm_whole", ctypes.c_int32), ("sink", ctypes.c_int32),
+                ("decay_channels", ctypes.c_int32), ("gate_rank", ctypes.c_int32), ("gate_act", ctypes.c_int32),
+                ("w_gate2", ctypes.c_void_p), ("a_log", ctypes.c_void_p), ("dt_bias", ctypes.c_void_p)]
 
 
 class HybridRunC(ctypes.Structure):
@@ -177,7 +203,7 @@ class HybridConfigC(ctypes.Structure):
                                               "max_batch", "max_out", "max_pages", "max_seq_len")] + [("eps", ctypes.c_float)] + \
                [("norm_kind", ctypes.c_int32), ("norm_groups", ctypes.c_int32), ("embed_scale", ctypes.c_float),
                 ("logit_softcap", ctypes.c_float), ("bigram_buckets", ctypes.c_int32), ("bigram_mul_prev", ctypes.c_int32),
-                ("bigram_mul_cur", ctypes.c_int32)]
+                ("bigram_mul_cur", ctypes.c_int32), ("logit_scale", ctypes.c_float)]
 
 
 class HybridWeightsC(ctypes.Structure):
@@ -197,7 +223,7 @@ def rotary_frequencies(rot_dims: int, base: float, factor: float) -> torch.Tenso
     return torch.pow(torch.tensor(base, dtype=torch.float32), -(2.0 * i) / rot_dims) / factor
 
 
-ROTARY_KINDS = ("attention", "latent_attention", "retention")
+ROTARY_KINDS = ("attention", "latent_attention", "retention", "causal_attention")
 
 
 def reduced_bigram(bigram) -> tuple:
@@ -214,7 +240,8 @@ def reduced_bigram(bigram) -> tuple:
 class HybridEngine(Qwen3Engine):
     """`weights`: {"embedding", "head", "final_norm", "loop_in" (or None), "layers": [per layer dict with norm1, norm2, w_in,
     b_in, w_out, lower, head_norm, w_up, w_down, b_up, b_down; per mixer kind also q_norm, k_norm | conv_w, conv_b, w_gates, b_gates,
-    lam | shift_mu, w_decay2, decay0, bonus | w_uq, w_ukT, w_uv, q_lat_norm, kv_lat_norm; "moe": {router, correction, w_gate_up,
+    lam | shift_mu, w_decay2, decay0, bonus | w_uq, w_ukT, w_uv, q_lat_norm, kv_lat_norm | conv_w, w_decay2, w_gate2, a_log, dt_bias
+    (delta rule); ls1, ls2 (layer scale); "moe": {router, router_bias, correction, w_gate_up (up rows only in the up / down form),
     w_down, shared_gate_up, shared_down}; "side": the same mixer keys for a sibling mixer], "bigram" (or None)} — matrices in any
     float dtype (stored as the engine's dtype), vectors and the router stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
 
@@ -249,6 +276,10 @@ class HybridEngine(Qwen3Engine):
             self._keep.append(t.to(dev, torch.float32).contiguous())
             return self._keep[-1].data_ptr()
 
+        def norm_w(t):
+            """A norm weight of the residual stream: stored around zero when the config says so (1 + w, formed in fp32)."""
+            return vec(t.float() + 1.0) if (t is not None and cfg.norm_one_plus) else vec(t)
+
         W = cfg.width
         sides = [(i, m.side) for i, m in enumerate(cfg.layers) if m.side is not None]
         larr = (HybridLayerC * (len(cfg.layers) + len(sides)))()
@@ -259,7 +290,11 @@ class HybridEngine(Qwen3Engine):
             assert tuple(lw["w_out"].shape) == (W, m.heads * m.vdim), (i, m.kind, tuple(lw["w_out"].shape))
             c.kind, c.heads, c.kv_heads, c.dim, c.vdim = MIXER_KINDS[m.kind], m.heads, m.kv_heads, m.dim, m.vdim
             c.window, c.pool, c.rot_dims, c.scale, c.gate_cap, c.ff = m.window, m.pool, m.rot_dims, m.scale, m.gate_cap, m.ff
-            c.norm1, c.norm2 = vec(lw["norm1"]), vec(lw.get("norm2"))
+            c.norm1, c.norm2 = norm_w(lw["norm1"]), norm_w(lw.get("norm2"))
+            c.ls1, c.ls2 = vec(lw.get("ls1")), vec(lw.get("ls2"))
+            c.qk_norm_whole, c.sink = int(m.qk_norm_whole), int(m.sink)
+            c.decay_channels, c.gate_rank, c.gate_act = int(m.decay_channels), m.gate_rank, GATE_KINDS[m.gate_act]
+            c.w_gate2, c.a_log, c.dt_bias = mat(lw.get("w_gate2")), vec(lw.get("a_log")), vec(lw.get("dt_bias"))
             c.w_in, c.b_in, c.w_out = mat(lw["w_in"]), vec(lw.get("b_in")), mat(lw["w_out"])
             c.lower, c.head_norm = vec(lw.get("lower")), vec(lw.get("head_norm"))
             c.inv_freq = vec(rotary_frequencies(m.rot_dims, m.rot_base, m.rot_factor)) if m.kind in ROTARY_KINDS and m.rot_dims else None
@@ -285,7 +320,8 @@ class HybridEngine(Qwen3Engine):
                 mc = HybridMoEC(e.experts, e.identity, e.top, e.ff, e.shared_ff, e.limit, e.shared_limit, e.act_alpha,
                                 vec(ew["router"]), vec(ew.get("correction")), mat(ew.get("w_gate_up")), mat(ew.get("w_down")),
                                 mat(ew.get("shared_gate_up")), mat(ew.get("shared_down")), ROUTER_SCORES[e.score], int(e.renorm),
-                                int(e.scale_input), e.up_offset)
+                                int(e.scale_input), e.up_offset, EXPERT_FORMS[e.expert_form], ACT_KINDS[e.expert_act],
+                                vec(ew.get("router_bias")) if e.router_bias else None)
                 self._moes.append(mc)
                 c.moe = ctypes.pointer(mc)
 
@@ -308,6 +344,11 @@ class HybridEngine(Qwen3Engine):
                     pool = torch.zeros(max_pages, (page_size - 1) // m.pool + 1, m.kv_heads, m.dim + m.vdim, dtype=torch.float32, device=dev)
                     self.pools.append(pool)
                     return kv.data_ptr(), pool.data_ptr(), None
+                if m.state_floats(W):
+                    # what the attention keeps per request besides its pages (the history of a convolution in front of it)
+                    st = torch.zeros(self.state_slots, m.state_floats(W), dtype=torch.float32, device=dev)
+                    self.states.append(st)
+                    return kv.data_ptr(), None, st.data_ptr()
                 return kv.data_ptr(), None, None
             st = torch.zeros(self.state_slots, m.state_floats(W), dtype=torch.float32, device=dev)
             self.states.append(st)
@@ -315,7 +356,8 @@ class HybridEngine(Qwen3Engine):
 
         for j, (li, loop_in) in enumerate(runs):
             m = cfg.layers[li]
-            rarr[j].layer, rarr[j].loop_in = li, int(loop_in)
+            # a loop without an input matrix just runs the range again: nothing happens between the passes
+            rarr[j].layer, rarr[j].loop_in = li, int(loop_in and weights.get("loop_in") is not None)
             rarr[j].cache, rarr[j].pool, rarr[j].state = storage(m)
             if m.side is not None:
                 rarr[j].side_cache, rarr[j].side_pool, rarr[j].side_state = storage(m.side)
@@ -323,7 +365,7 @@ class HybridEngine(Qwen3Engine):
         bg = reduced_bigram(cfg.bigram)
         cc = HybridConfigC(W, cfg.vocab, len(larr), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
                            max_batch, self.max_out, max_pages, max_seq_len, cfg.eps, NORM_KINDS[cfg.norm_kind], cfg.norm_groups,
-                           cfg.embed_scale, cfg.logit_softcap, int(bg[0]), int(bg[1]), int(bg[2]))
+                           cfg.embed_scale, cfg.logit_softcap, int(bg[0]), int(bg[1]), int(bg[2]), float(cfg.logit_scale))
         # the last token every state slot's sequence has seen (what a bigram embedding needs of the step before)
         self.prev_token = torch.zeros(self.state_slots, dtype=torch.int32, device=dev)
         if cfg.bigram and tuple(weights["bigram"].shape) != (int(bg[0]) + 1, W):
@@ -331,7 +373,7 @@ class HybridEngine(Qwen3Engine):
         emb = mat(weights["embedding"])
         head = emb if weights["head"] is weights["embedding"] else mat(weights["head"])      # a tied head shares the table
         cw = HybridWeightsC(ctypes.cast(larr, ctypes.POINTER(HybridLayerC)), ctypes.cast(rarr, ctypes.POINTER(HybridRunC)),
-                            emb, mat(weights.get("loop_in")), head, vec(weights["final_norm"]),
+                            emb, mat(weights.get("loop_in")), head, norm_w(weights["final_norm"]),
                             mat(weights.get("bigram")) if cfg.bigram else None, self.prev_token.data_ptr())
         self._larr, self._rarr = larr, rarr
         h = ctypes.c_void_p()
