@@ -197,6 +197,12 @@ def _dipivik(model_name, device="cuda:0", weights=None, checkpoint_dir=None, syn
     return _hybrid_lm(".dipivik", "DipivikModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
 
 
+@register_model("sizitar")
+def _sizitar(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
+    """Looped sequential LM of gated delta-rule layers and sink attention behind short convolutions, with layer scale and relu-squared experts."""
+    return _hybrid_lm(".sizitar", "SizitarModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
+
+
 def load_checkpoint_dir(path: str, device: str = "cuda:0", **kw):
     """A local checkpoint folder whose config.json names its architecture: the registry entry of that name loads it."""
     import json
