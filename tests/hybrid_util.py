@@ -1,4 +1,4 @@
-"""Helpers of the hybrid-engine tests (Sirodra, Fusanex, Dipivik): small configurations, random checkpoints, and a driver that feeds token
+"""Helpers of the hybrid-engine tests (Sirodra, Fusanex, Dipivik, Sizitar): small configurations, random checkpoints, and a driver that feeds token
 portions through ModelWorker the way a serving step does."""
 import math
 
@@ -70,8 +70,8 @@ class Driver:
         from vox_serve_amd.model import get_model_class
         from vox_serve_amd.worker.base import ModelWorker
         # the registry entry of the config's architecture builds the model, as for a checkpoint folder
-        from vox_serve_amd.model import dipivik, fusanex, sirodra
-        mod = {"Sirodra": sirodra, "Fusanex": fusanex, "Dipivik": dipivik}[cfg["architecture"]]
+        from vox_serve_amd.model import dipivik, fusanex, sirodra, sizitar
+        mod = {"Sirodra": sirodra, "Fusanex": fusanex, "Dipivik": dipivik, "Sizitar": sizitar}[cfg["architecture"]]
         self.model = get_model_class(cfg["architecture"])(cfg["architecture"].lower() + "-test", weights=S, config=mod.config_from_dict(cfg),
                                                           dtype=dtype, max_batch_size=max_batch, page_size=page_size, max_num_pages=pages,
                                                           max_seq_len=pages * page_size, max_prefill_tokens=max_rows,
