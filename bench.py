@@ -749,8 +749,15 @@ def main():
     ap.add_argument("--fusanex", action="store_true", help="instead of the default workload: prefill / decode throughput of the Fusanex "
                     "design (random weights) beside Sirodra, the closest existing model, on the same engine at equal width and depth "
                     "(tools/bench_fusanex.py); prints that comparison as one JSON line")
+    ap.add_argument("--sizitar", action="store_true", help="instead of the default workload: prefill / decode throughput of the Sizitar "
+                    "design (random weights) beside Fusanex, the closest existing model, on the same engine at equal width and depth "
+                    "(tools/bench_sizitar.py); prints that comparison as one JSON line")
     args = ap.parse_args()
 
+    if args.sizitar:
+        from tools.bench_sizitar import run as run_sizitar
+        print(json.dumps(run_sizitar(steps=min(args.steps, 50), warmup=min(args.warmup, 10))))
+        return
     if args.dipivik:
         from tools.bench_dipivik import run as run_dipivik
         print(json.dumps(run_dipivik(steps=min(args.steps, 50), warmup=min(args.warmup, 10))))
