@@ -574,19 +574,23 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
 // times from cache instead of once from a normalised copy, and a dependent launch is saved.  Needs K % 8 == 0 (4 for fp32).
 template <typename T, int EPI, int CPW>
 __global__ __launch_bounds__(256) void k_hb_ln_gemv(const float* X, long ldx, const int* rows, const float* lnw, float eps, const T* Wt,
-                                                    const float* bias, float* C, int N, int K) {
+                                                    const float* bias, float* C, int N, int K, int rms, float epi_arg) {
     const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CPW;
     if (n0 >= N) return;
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     const float* xr = X + (size_t)(rows ? rows[0] : 0) * ldx;
-    float s = 0.f;
-    for (int k = lane * CH; k < K; k += 64 * CH)
+    // rms != 0: the RMS norm over the whole row (no mean is taken off)
+    float mean = 0.f;
+    if (!rms) {
+        float s = 0.f;
+        for (int k = lane * CH; k < K; k += 64 * CH)
 #pragma unroll
-        for (int e = 0; e < CH; e += 4) {
-            const float4 x4 = *(const float4*)(xr + k + e);
-            s += x4.x; s += x4.y; s += x4.z; s += x4.w;
-        }
-    const float mean = hb_wave_sum(s) / (float)K;
+            for (int e = 0; e < CH; e += 4) {
+                const float4 x4 = *(const float4*)(xr + k + e);
+                s += x4.x; s += x4.y; s += x4.z; s += x4.w;
+            }
+        mean = hb_wave_sum(s) / (float)K;
+    }
     float q = 0.f;
     for (int k = lane * CH; k < K; k += 64 * CH)
 #pragma unroll
@@ -632,23 +636,25 @@ __global__ __launch_bounds__(256) void k_hb_ln_gemv(const float* X, long ldx, co
 #pragma unroll
     for (int j = 0; j < CPW; ++j) {
         const float sum = hb_wave_sum(acc[j]);
-        if (n0 + j < N && lane == 0) hb_epilogue<EPI>(C + n0 + j, sum, bias ? bias[n0 + j] : 0.f);
+        if (n0 + j < N && lane == 0) hb_epilogue<EPI>(C + n0 + j, sum, bias ? bias[n0 + j] : 0.f, epi_arg);
     }
 }
 // true: the fused form was launched (one row, aligned operands); false: the caller normalises and multiplies in two launches
 template <typename T>
 bool hb_try_ln_gemv(hipStream_t st, int epi, const float* X, long ldx, const int* rows, const float* lnw, float eps, const T* W, const float* bias,
-                    float* C, int N, int K) {
+                    float* C, int N, int K, int rms = 0, float epi_arg = 0.f) {
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     if (K % CH || (ldx & 3) || ((size_t)X & 15) || ((size_t)W & 15) || ((size_t)lnw & 15)) return false;
     const bool wide = N >= 16 * 1024;
     const dim3 g(wide ? (N + 15) / 16 : (N + 3) / 4), b(256);
 #define HB_LN(EPI_) \
     do { \
-        if (wide) hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 4>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K); \
-        else hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 1>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K); \
+        if (wide) hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 4>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K, rms, epi_arg); \
+        else hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 1>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K, rms, epi_arg); \
     } while (0)
     if (epi == HB_EPI_GELU) HB_LN(HB_EPI_GELU);
+    else if (epi == HB_EPI_SCALE) HB_LN(HB_EPI_SCALE);
+    else if (epi != HB_EPI_STORE) return false;
     else HB_LN(HB_EPI_STORE);
 #undef HB_LN
     return true;
@@ -3209,11 +3215,12 @@ static void hb_norm(const vox_hybrid* m, hipStream_t st, int n, const float* x, 
         if (w2) hb_layernorm(st, n, x, ldx, rows, w2, y2, ldy, c.width, c.eps);
     }
 }
-// the fused one-row norm + GEMV exists for the layer norm only
+// the fused one-row norm + GEMV exists for the layer norm and for the RMS norm over one slice
 template <typename T>
 static bool hb_try_norm_gemv(const vox_hybrid* m, hipStream_t st, int epi, const float* X, long ldx, const int* rows, const float* nw, const T* W,
-                             const float* bias, float* C, int N, int K) {
-    return m->cfg.norm_kind == VOX_NORM_LAYER && hb_try_ln_gemv<T>(st, epi, X, ldx, rows, nw, m->cfg.eps, W, bias, C, N, K);
+                             const float* bias, float* C, int N, int K, float epi_arg = 0.f) {
+    const bool rms = m->cfg.norm_kind == VOX_NORM_RMS_GROUPS && m->cfg.norm_groups == 1;
+    return (m->cfg.norm_kind == VOX_NORM_LAYER || rms) && hb_try_ln_gemv<T>(st, epi, X, ldx, rows, nw, m->cfg.eps, W, bias, C, N, K, rms ? 1 : 0, epi_arg);
 }
 
 // The matrix-core latent attention for steps of many rows over a bf16 cache.  false: the shapes do not fit it (rows of the cache that are
@@ -3646,10 +3653,11 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        if (!(n_out == 1 && !(c.logit_softcap > 0.f) && (c.logit_scale == 0.f || c.logit_scale == 1.0f) &&
-              hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr, io->logits, c.vocab, W))) {
+        const bool scaled = c.logit_scale != 0.f && c.logit_scale != 1.0f;
+        if (!(n_out == 1 && !(c.logit_softcap > 0.f) &&
+              hb_try_norm_gemv<T>(m, st, scaled ? HB_EPI_SCALE : HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr,
+                                  io->logits, c.vocab, W, c.logit_scale))) {
             hb_norm(m, st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, nullptr, nullptr, (long)W);
-            const bool scaled = c.logit_scale != 0.f && c.logit_scale != 1.0f;
             hb_rowmap rm = hb_plain();
             rm.epi_arg = c.logit_softcap > 0.f ? c.logit_softcap : c.logit_scale;
             VOX_TRY(hb_gemm<T>(st, c.logit_softcap > 0.f ? HB_EPI_SOFTCAP : (scaled ? HB_EPI_SCALE : HB_EPI_STORE), m->hout, W, (const T*)m->w.head,
